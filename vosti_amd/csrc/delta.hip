@@ -90,6 +90,19 @@ __global__ __launch_bounds__(256) void delta_decay_kernel(float* __restrict__ g,
   g[e] = expf(-expf(load_weight(A_log, w_is_f32, col / d)) * sp);
 }
 
+// g[t, c] = sigmoid(a[t, c] + bias[c])^inv_root, as exp(-softplus(-z) * inv_root): the logarithm of the logistic function
+// is -softplus(-z), so the power needs no logarithm of a number near 1.
+__global__ __launch_bounds__(256) void gla_decay_kernel(float* __restrict__ g, const elem_t* __restrict__ a, int64_t lda, const void* __restrict__ bias,
+                                                        int w_is_f32, int HD, float inv_root, int64_t numel) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= numel) return;
+  const int64_t t = e / HD;
+  const int col = (int)(e - t * HD);
+  const float z = -(to_f32(a[t * lda + col]) + load_weight(bias, w_is_f32, col));
+  const float sp = z > 20.f ? z : log1pf(expf(z));
+  g[e] = expf(-sp * inv_root);
+}
+
 // The two unit norms and the decays of a token in one launch: workgroup (token, j) is q's head j, k's head j - G, or
 // the decays of head j - 2 G; the arithmetic is delta_unit_kernel's and delta_decay_kernel's.
 __global__ __launch_bounds__(64) void delta_prep_kernel(float* x, int64_t ld, int q_col, int k_col, int G, int H, int d, float unit_eps,
@@ -138,12 +151,15 @@ struct RuleShape {
   static constexpr int NV = (TC * CB + RULE_THREADS - 1) / RULE_THREADS;
 };
 
-template <int R, int DR>
-__global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qkv, int64_t ld, int q_col,
+//
+// DELTA false is the same walk without the correction: S <- diag(g) S + k v^T; o = S^T q (gated linear attention); beta is
+// not read, q is multiplied by q_scale as it is brought in, and the inputs may be elements (IN).
+template <int R, int DR, bool DELTA, typename IN>
+__global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restrict__ out, const IN* __restrict__ qkv, int64_t ld, int q_col,
                                                                   int k_col, int v_col, const float* __restrict__ decay,
                                                                   const elem_t* __restrict__ b, int64_t ldb, float* state, int64_t state_stride,
                                                                   const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
-                                                                  const int32_t* __restrict__ slots, int H, int G, int d, int dv) {
+                                                                  const int32_t* __restrict__ slots, int H, int G, int d, int dv, float q_scale) {
   using Sh = RuleShape<R, DR>;
   constexpr int DMAX = Sh::DMAX, TC = Sh::TC, CB = Sh::CB;
   __shared__ __attribute__((aligned(16))) float smem[2 * Sh::BUF];
@@ -189,10 +205,10 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
       const bool ok = e < TC * DMAX && t0 + tok < n && c < d;
       const int64_t t = first + t0 + (ok ? tok : 0);
       const int cc = ok ? c : 0;
-      const float kv = qkv[t * ld + k_col + (int64_t)g * d + cc], qv = qkv[t * ld + q_col + (int64_t)g * d + cc];
+      const float kv = to_f32(qkv[t * ld + k_col + (int64_t)g * d + cc]), qv = to_f32(qkv[t * ld + q_col + (int64_t)g * d + cc]);
       const float gv = decay[(t * H + h) * d + cc];
       pk[it] = ok ? kv : 0.f;
-      pq[it] = ok ? qv : 0.f;
+      pq[it] = ok ? (DELTA ? qv : qv * q_scale) : 0.f;
       pg[it] = ok ? gv : 1.f;
     }
 #pragma unroll
@@ -201,10 +217,10 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
       const int tok = e / CB, c = e - tok * CB;
       const bool ok = e < TC * CB && t0 + tok < n && blockIdx.z * CB + c < dv;
       const int64_t t = first + t0 + (ok ? tok : 0);
-      const float vv = qkv[t * ld + v_col + (int64_t)h * dv + (ok ? blockIdx.z * CB + c : 0)];
+      const float vv = to_f32(qkv[t * ld + v_col + (int64_t)h * dv + (ok ? blockIdx.z * CB + c : 0)]);
       pv[it] = ok ? vv : 0.f;
     }
-    if (tid < TC) {
+    if (DELTA && tid < TC) {
       const bool ok = t0 + tid < n;
       const float bb = to_f32(b[(int64_t)(first + t0 + (ok ? tid : 0)) * ldb + h]);
       pb = ok ? sigmoid_f(bb) : 0.f;
@@ -267,10 +283,12 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
       }
       if (tok + 1 < here) read(tok + 1);
       // Fused multiply-adds, written out: one instruction and one rounding a step.
+      if (DELTA) {
 #pragma unroll
-      for (int i = 0; i < DR; ++i) dot = __builtin_fmaf(S[i], kk[i], dot);
-      dot = group_sum<R>(dot);
-      const float u = beta * (v - dot);
+        for (int i = 0; i < DR; ++i) dot = __builtin_fmaf(S[i], kk[i], dot);
+        dot = group_sum<R>(dot);
+      }
+      const float u = DELTA ? beta * (v - dot) : v;
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < DR; ++i) {
@@ -296,18 +314,19 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
   }
 }
 
-// y[t, h, :] = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t, h, :]), stored as elements in rows of length ldy; the
+// y[t, h, :] = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t, h, :]) (gate_kind 1: * silu(gate[t, h, :])), stored as elements in rows of length ldy; the
 // columns beyond the heads are set to zero (a projection with padded columns reads them).  One wave per (token, head).
 __global__ __launch_bounds__(64) void delta_out_kernel(elem_t* __restrict__ y, int64_t ldy, const float* __restrict__ o,
                                                        const elem_t* __restrict__ gate, int64_t ldg, const void* __restrict__ w, int w_is_f32,
-                                                       int H, int dv, float eps) {
+                                                       int H, int dv, float eps, int gate_kind) {
   const int t = blockIdx.x / H, h = blockIdx.x - t * H;
   const float* row = o + ((int64_t)t * H + h) * dv;
   float part = 0.f;
   for (int c = threadIdx.x; c < dv; c += 64) part = part + row[c] * row[c];
   const float rr = rsqrtf(wave_sum_xor(part) / (float)dv + eps);
   for (int c = threadIdx.x; c < dv; c += 64) {
-    const float gt = sigmoid_f(to_f32(gate[(int64_t)t * ldg + (int64_t)h * dv + c]));
+    const float gz = to_f32(gate[(int64_t)t * ldg + (int64_t)h * dv + c]);
+    const float gt = gate_kind == 0 ? sigmoid_f(gz) : silu_f(gz);
     y[(int64_t)t * ldy + (int64_t)h * dv + c] = from_f32<elem_t>(((row[c] * rr) * load_weight(w, w_is_f32, c)) * gt);
   }
   if (h == H - 1)
@@ -386,9 +405,11 @@ int vk_delta_prep(float* x, int64_t ld, int q_col, int k_col, int T, int G, int 
 // out [T, H, dv] floats.  qkv: float rows of length ld with q (G heads of d) at q_col, k at k_col, v (H heads of dv) at
 // v_col; decay [T, H, d] floats; b: elements, beta's pre-activation of head h at b[t * ldb + h].  state: per slot,
 // the H states at its start, each [dv][d].
-int vk_delta_rule(float* out, const float* qkv, int64_t ld, int q_col, int k_col, int v_col, const float* decay, const elem_t* b, int64_t ldb,
-                  float* state, int64_t state_stride, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int G,
-                  int d, int dv, hipStream_t st) {
+extern "C++" {
+template <bool DELTA, typename IN>
+static int rule_launch(float* out, const IN* qkv, int64_t ld, int q_col, int k_col, int v_col, const float* decay, const elem_t* b, int64_t ldb,
+                       float* state, int64_t state_stride, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int G,
+                       int d, int dv, float q_scale, hipStream_t st) {
   VK_REQUIRE(S >= 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0, "delta rule: bad sizes H=%d G=%d d=%d dv=%d", H, G, d, dv);
   VK_REQUIRE(d <= 1024, "delta rule: key size %d exceeds 1024", d);
   VK_REQUIRE(state_stride >= (int64_t)H * d * dv, "delta rule: the state is too small");
@@ -398,7 +419,7 @@ int vk_delta_rule(float* out, const float* qkv, int64_t ld, int q_col, int k_col
   const dim3 grid(S, H, (dv + cols - 1) / cols);
   VK_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "delta rule: too many heads or columns");
 #define RULE(RR, DD) \
-  delta_rule_kernel<RR, DD><<<grid, RULE_THREADS, 0, st>>>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, H, G, d, dv)
+  delta_rule_kernel<RR, DD, DELTA, IN><<<grid, RULE_THREADS, 0, st>>>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, H, G, d, dv, q_scale)
   if (DR == 4) {
     switch (R) {
       case 1: RULE(1, 4); break;
@@ -417,14 +438,51 @@ int vk_delta_rule(float* out, const float* qkv, int64_t ld, int q_col, int k_col
 #undef RULE
   return vk_check_launch("delta rule");
 }
+}  // extern "C++"
+
+int vk_delta_rule(float* out, const float* qkv, int64_t ld, int q_col, int k_col, int v_col, const float* decay, const elem_t* b, int64_t ldb,
+                  float* state, int64_t state_stride, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int G,
+                  int d, int dv, hipStream_t st) {
+  return rule_launch<true, float>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, S, H, G, d, dv, 1.f,
+                                  st);
+}
+
+// Gated linear attention: g [T, H, d] = sigmoid(a + bias)^(1 / root) = exp(-softplus(-(a + bias)) / root) from the
+// elements a (rows of length lda) and the bias [H d], in 32-bit.
+int vk_gla_decay(float* g, const elem_t* a, int64_t lda, const void* bias, int w_is_f32, int T, int HD, float root, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && HD > 0 && lda >= HD && root > 0.f, "linear attention decay: bad sizes T=%d channels=%d root=%g", T, HD, (double)root);
+  const int64_t numel = (int64_t)T * HD;
+  if (numel == 0) return 0;
+  gla_decay_kernel<<<(unsigned)((numel + 255) / 256), 256, 0, st>>>(g, a, lda, bias, w_is_f32, HD, 1.f / root, numel);
+  return vk_check_launch("linear attention decay");
+}
+
+// The recurrence S <- diag(g) S + k v^T, o = S^T (q * q_scale) per head.  x: element rows of length ld with q (H heads of
+// d) at q_col, k at k_col, v (H heads of dv) at v_col; decay [T, H, d] floats; out [T, H, dv] floats; state as vk_delta_rule's.
+int vk_gla_rule(float* out, const elem_t* x, int64_t ld, int q_col, int k_col, int v_col, const float* decay, float* state, int64_t state_stride,
+                const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int d, int dv, float q_scale, hipStream_t st) {
+  return rule_launch<false, elem_t>(out, x, ld, q_col, k_col, v_col, decay, nullptr, 0, state, state_stride, cu_q, positions, slots, S, H, H, d, dv,
+                                    q_scale, st);
+}
 
 int vk_delta_out(elem_t* y, int64_t ldy, const float* o, const elem_t* gate, int64_t ldg, const void* w, int w_is_f32, int T, int H, int dv,
                  float eps, hipStream_t st) {
   VK_REQUIRE(T >= 0 && H > 0 && dv > 0 && ldg >= (int64_t)H * dv && ldy >= (int64_t)H * dv, "delta read-out: bad sizes");
   if (T == 0) return 0;
   VK_REQUIRE((int64_t)T * H < (1ll << 31), "delta read-out: too many rows");
-  delta_out_kernel<<<T * H, 64, 0, st>>>(y, ldy, o, gate, ldg, w, w_is_f32, H, dv, eps);
+  delta_out_kernel<<<T * H, 64, 0, st>>>(y, ldy, o, gate, ldg, w, w_is_f32, H, dv, eps, 0);
   return vk_check_launch("delta read-out");
+}
+
+// The same read-out with a choice of gate: gate_kind 0 is the logistic function of the gate's input, 1 is z * logistic(z).
+int vk_gated_head_norm(elem_t* y, int64_t ldy, const float* o, const elem_t* gate, int64_t ldg, const void* w, int w_is_f32, int T, int H, int dv,
+                       float eps, int gate_kind, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && H > 0 && dv > 0 && ldg >= (int64_t)H * dv && ldy >= (int64_t)H * dv && (gate_kind == 0 || gate_kind == 1),
+             "gated head norm: bad sizes");
+  if (T == 0) return 0;
+  VK_REQUIRE((int64_t)T * H < (1ll << 31), "gated head norm: too many rows");
+  delta_out_kernel<<<T * H, 64, 0, st>>>(y, ldy, o, gate, ldg, w, w_is_f32, H, dv, eps, gate_kind);
+  return vk_check_launch("gated head norm");
 }
 
 }  // extern "C"

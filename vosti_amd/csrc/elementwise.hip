@@ -252,6 +252,32 @@ __global__ __launch_bounds__(512) void pull_kernel(const u32x4* __restrict__ p, 
 }
 
 // ================================================================ host side
+// x[t, c] <- x[t, c] * act(gate[t, c]) for c < W, the product in 32-bit and rounded once: act is the logistic function
+// (kind 0) or z * logistic(z) (kind 1).  The gate's rows may be columns of a wider tensor (ldg).  A thread takes a
+// 16-byte vector when rows and strides are whole vectors (vec), an element otherwise.
+__device__ __forceinline__ float gate_value(float z, int kind) {
+  const float s = 1.f / (1.f + expf(-z));
+  return kind == 0 ? s : z * s;
+}
+__global__ __launch_bounds__(256) void gate_mul_kernel(elem_t* x, int64_t ldx, const elem_t* __restrict__ gate, int64_t ldg, int T, int W, int kind,
+                                                       int vec) {
+  const int per = vec ? W / VK_VEC : W;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)T * per) return;
+  const int64_t t = i / per;
+  const int c = (int)(i - t * per);
+  if (vec) {
+    float xv[VK_VEC], gv[VK_VEC];
+    load_elems(x + t * ldx + (int64_t)c * VK_VEC, xv);
+    load_elems(gate + t * ldg + (int64_t)c * VK_VEC, gv);
+#pragma unroll
+    for (int j = 0; j < VK_VEC; ++j) xv[j] = xv[j] * gate_value(gv[j], kind);
+    store_elems(x + t * ldx + (int64_t)c * VK_VEC, xv);
+  } else {
+    x[t * ldx + c] = from_f32<elem_t>(to_f32(x[t * ldx + c]) * gate_value(to_f32(gate[t * ldg + c]), kind));
+  }
+}
+
 extern "C" {
 
 int vk_embedding(elem_t* out, const elem_t* table, const int32_t* ids, int T, int H, int V, hipStream_t st) {
@@ -368,6 +394,15 @@ int vk_fill_random(elem_t* out, int64_t n, uint64_t seed, int kind, float p0, fl
   VK_REQUIRE((n + 255) / 256 <= 0x7fffffff, "fill_random: tensor too large");
   fill_random_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(out, n, seed, kind, p0, p1);
   return vk_check_launch("fill_random");
+}
+
+int vk_gate_mul(elem_t* x, int64_t ldx, const elem_t* gate, int64_t ldg, int T, int W, int kind, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && W > 0 && ldx >= W && ldg >= W && (kind == 0 || kind == 1), "gate: bad sizes T=%d W=%d kind=%d", T, W, kind);
+  if (T == 0) return 0;
+  const int vec = W % VK_VEC == 0 && ldx % VK_VEC == 0 && ldg % VK_VEC == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)gate % 16 == 0;
+  const int64_t n = (int64_t)T * (vec ? W / VK_VEC : W);
+  gate_mul_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(x, ldx, gate, ldg, T, W, kind, vec);
+  return vk_check_launch("gate");
 }
 
 }  // extern "C"

@@ -130,9 +130,19 @@ struct Kernels::Fn {
   int (*moe_down)(P, CP, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
   int (*moe_combine)(P, CP, CP, CP, int, int, int, hipStream_t);
   int (*moe_relu_square)(P, int64_t, hipStream_t);
+  int (*qkv_post_norm_angles)(CP, int64_t, P, P, P, CP, CP, int, int, float, CP, float, int, CP, CP, int, int, int, int, int, hipStream_t);
+  int (*gate_mul)(P, int64_t, CP, int64_t, int, int, int, hipStream_t);
+  int (*gla_decay)(P, CP, int64_t, CP, int, int, int, float, hipStream_t);
+  int (*gla_rule)(P, CP, int64_t, int, int, int, CP, P, int64_t, CP, CP, CP, int, int, int, int, float, hipStream_t);
+  int (*gated_head_norm)(P, int64_t, CP, CP, int64_t, CP, int, int, int, int, float, int, hipStream_t);
+  int (*moe_route_bias)(P, P, P, CP, CP, CP, int, int, int, int, int, float, hipStream_t);
+  int (*moe_up_plain)(P, int64_t, CP, int64_t, CP, CP, CP, CP, int, int, int, int, int, hipStream_t);
+  int (*moe_glu)(P, CP, int64_t, int, float, float, float, hipStream_t);
+  int (*moe_combine_add)(P, CP, CP, CP, CP, int, int, int, hipStream_t);
+  int (*stream_norm_add_f32)(P, CP, CP, CP, int, int, int, float, float, float, hipStream_t);
 };
 
-static constexpr int KERNEL_ABI = 16;
+static constexpr int KERNEL_ABI = 17;
 
 Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(name), fn_(new Fn) {
   if (name == "bf16") dtype_ = DType::BF16;
@@ -167,6 +177,9 @@ Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(na
   VK(stream_pair_norm, "vk_stream_pair_norm"); VK(ssm_scan, "vk_ssm_scan"); VK(ssm_gate_norm, "vk_ssm_gate_norm");
   VK(moe_max_tiles, "vk_moe_max_tiles"); VK(moe_route, "vk_moe_route"); VK(moe_plan, "vk_moe_plan"); VK(moe_up, "vk_moe_up");
   VK(moe_down, "vk_moe_down"); VK(moe_combine, "vk_moe_combine"); VK(moe_relu_square, "vk_moe_relu_square"); VK(gemm_grouped, "vk_gemm_grouped");
+  VK(qkv_post_norm_angles, "vk_qkv_post_norm_angles"); VK(gate_mul, "vk_gate_mul"); VK(gla_decay, "vk_gla_decay"); VK(gla_rule, "vk_gla_rule");
+  VK(gated_head_norm, "vk_gated_head_norm"); VK(moe_route_bias, "vk_moe_route_bias"); VK(moe_up_plain, "vk_moe_up_plain"); VK(moe_glu, "vk_moe_glu");
+  VK(moe_combine_add, "vk_moe_combine_add"); VK(stream_norm_add_f32, "vk_stream_norm_add_f32");
 #undef VK
   segment_keys_ = fn_->attn_segment_keys();
   item_rows_ = fn_->attn_item_rows();
@@ -449,11 +462,16 @@ Tensor Kernels::stream_norm(const Tensor& x, const Tensor& w, float eps, float o
 }
 
 void Kernels::stream_norm_add(Tensor& out, const Tensor& base, const Tensor& y, const Tensor& w, float eps, float offset, float mult) {
-  expect(y, "norm input", dtype_);
+  if (y.dtype != DType::F32) expect(y, "norm input", dtype_);
   if (y.shape.size() != 2) throw EngineError("norm input is " + y.describe());
   expect(base, "stream", DType::F32, y.shape);
   expect(out, "stream", DType::F32, y.shape);
   const int wf = norm_weight(w, "norm weight", y.dim(1));
+  // A sublayer's rows may be elements or, where it left them unrounded, floats.
+  if (y.dtype == DType::F32 && dtype_ != DType::F32) {
+    call(fn_->stream_norm_add_f32(out.data, base.data, y.data, w.data, wf, (int)y.dim(0), (int)y.dim(1), eps, offset, mult, stream));
+    return;
+  }
   call(fn_->stream_norm_add(out.data, base.data, y.data, w.data, wf, (int)y.dim(0), (int)y.dim(1), eps, offset, mult, stream));
 }
 
@@ -700,6 +718,93 @@ Tensor Kernels::qkv_post_angles(const Tensor& qkv, int nq, int nkv, int d, const
   return q_out;
 }
 
+Tensor Kernels::qkv_post_norm_angles(const Tensor& qkv, int nq, int nkv, int d, const Tensor* k_cache, const Tensor* v_cache, int page_size,
+                                     const Tensor* q_w, const Tensor* k_w, int norm_d, float eps, const Tensor& inv_freq, float mag,
+                                     const Tensor& positions, const Tensor* slots) {
+  expect(qkv, "qkv", dtype_);
+  const int64_t W = (int64_t)(nq + 2 * nkv) * d;
+  if (qkv.shape.size() != 2 || qkv.dim(1) < W) throw EngineError("qkv_post: rows are " + qkv.describe() + ", expected a width of at least " + std::to_string(W));
+  const int64_t T = qkv.dim(0);
+  expect(inv_freq, "rotation frequencies", DType::F32);
+  if (norm_d < 1 || norm_d > d || inv_freq.shape.size() != 1 || inv_freq.dim(0) < 1 || 2 * inv_freq.dim(0) > norm_d)
+    throw EngineError("qkv_post: rotation frequencies are " + inv_freq.describe() + " for a head norm over " + std::to_string(norm_d) + " of " +
+                      std::to_string(d));
+  int wf = 0;
+  if (q_w) wf = norm_weight(*q_w, "q norm weight", norm_d);
+  if (k_w) {
+    const int wf2 = norm_weight(*k_w, "k norm weight", norm_d);
+    if (q_w && wf2 != wf) throw EngineError("qkv_post: q and k norm weights must have the same type");
+    wf = wf2;
+  }
+  expect(positions, "positions", DType::I32, {T});
+  Tensor q_out;
+  if (nq) q_out = empty({T, nq, d});
+  if (nkv) {
+    if (!k_cache || !v_cache || !slots) throw EngineError("qkv_post: a store needs both caches and slots");
+    if (k_cache->shape.size() != 4) throw EngineError("k cache is " + k_cache->describe());
+    const int64_t pages = k_cache->dim(0);
+    expect(*k_cache, "k cache", dtype_, {pages, nkv, page_size, d});
+    expect(*v_cache, "v cache", dtype_, {pages, nkv, d, page_size});
+    expect(*slots, "slots", DType::I32, {T});
+  }
+  call(fn_->qkv_post_norm_angles(qkv.data, qkv.dim(1), nq ? q_out.data : nullptr, nkv ? k_cache->data : nullptr, nkv ? v_cache->data : nullptr,
+                                 q_w ? q_w->data : nullptr, k_w ? k_w->data : nullptr, wf, norm_d, eps, inv_freq.data, mag, (int)inv_freq.dim(0),
+                                 positions.data, nkv ? slots->data : nullptr, (int)T, nq, nkv, d, page_size, stream));
+  return q_out;
+}
+
+void Kernels::gate_mul(Tensor& x, const Tensor& gate, int64_t gate_col, int kind) {
+  expect(x, "gated rows", dtype_);
+  expect(gate, "gate", dtype_);
+  if (x.shape.size() != 2 || gate.shape.size() != 2 || gate.dim(0) != x.dim(0) || gate_col < 0 || gate_col + x.dim(1) > gate.dim(1))
+    throw EngineError("gate: rows " + x.describe() + " with the gate's " + gate.describe() + " from column " + std::to_string(gate_col));
+  call(fn_->gate_mul(x.data, x.dim(1), static_cast<const char*>(gate.data) + (size_t)gate_col * dtype_bytes(dtype_), gate.dim(1), (int)x.dim(0),
+                     (int)x.dim(1), kind, stream));
+}
+
+// ------------------------------------------------------------------------- gated linear attention
+Tensor Kernels::gla_decay(const Tensor& a, const Tensor& bias, int H, int d, float root) {
+  expect(a, "decay input", dtype_);
+  if (a.shape.size() != 2 || a.dim(1) != (int64_t)H * d) throw EngineError("linear attention decay: input is " + a.describe());
+  const int wf = norm_weight(bias, "decay bias", (int64_t)H * d);
+  Tensor g = empty({a.dim(0), H, d}, DType::F32);
+  call(fn_->gla_decay(g.data, a.data, a.dim(1), bias.data, wf, (int)a.dim(0), H * d, root, stream));
+  return g;
+}
+
+Tensor Kernels::gla_rule(const Tensor& x, int64_t q_col, int64_t k_col, int64_t v_col, const Tensor& decay, Tensor& state, const Tensor& cu_q,
+                         const Tensor& positions, const Tensor& slots, int H, int d, int dv, float q_scale) {
+  expect(x, "linear attention input", dtype_);
+  expect(state, "state", DType::F32);
+  if (x.shape.size() != 2 || state.shape.size() != 2 || q_col < 0 || k_col < 0 || v_col < 0 || std::max(q_col, k_col) + (int64_t)H * d > x.dim(1) ||
+      v_col + (int64_t)H * dv > x.dim(1) || state.dim(1) < (int64_t)H * d * dv)
+    throw EngineError("linear attention: input " + x.describe() + ", state " + state.describe());
+  const int64_t T = x.dim(0), S = slots.numel();
+  expect(decay, "decay", DType::F32, {T, H, d});
+  expect(positions, "positions", DType::I32, {T});
+  expect(cu_q, "cu_q", DType::I32, {S + 1});
+  expect(slots, "state slots", DType::I32, {S});
+  Tensor out = empty({T, H, dv}, DType::F32);
+  call(fn_->gla_rule(out.data, x.data, x.dim(1), (int)q_col, (int)k_col, (int)v_col, decay.data, state.data, state.dim(1), cu_q.data, positions.data,
+                     slots.data, (int)S, H, d, dv, q_scale, stream));
+  return out;
+}
+
+Tensor Kernels::gated_head_norm(const Tensor& o, const Tensor& gate, int64_t gate_col, const Tensor& w, int H, int dv, float eps, int gate_kind,
+                                int64_t width) {
+  expect(o, "read-out", DType::F32);
+  expect(gate, "gate", dtype_);
+  if (o.shape.size() != 3 || o.dim(1) != H || o.dim(2) != dv || gate.shape.size() != 2 || gate.dim(0) != o.dim(0) || gate_col < 0 ||
+      gate_col + (int64_t)H * dv > gate.dim(1))
+    throw EngineError("gated head norm: " + o.describe() + " with gate " + gate.describe());
+  const int wf = norm_weight(w, "read-out norm weight", dv);
+  if (width < (int64_t)H * dv) throw EngineError("gated head norm: a row of " + std::to_string(width) + " does not hold the heads");
+  Tensor y = empty({o.dim(0), width});
+  call(fn_->gated_head_norm(y.data, width, o.data, static_cast<const char*>(gate.data) + (size_t)gate_col * dtype_bytes(dtype_), gate.dim(1), w.data, wf,
+                            (int)o.dim(0), H, dv, eps, gate_kind, stream));
+  return y;
+}
+
 // ---------------------------------------------------------------------------- state-space recurrence
 Tensor Kernels::ssm_scan(const Tensor& xbc, int64_t b_col, int64_t c_col, const Tensor& proj, int64_t dt_col, const Tensor& dt_bias,
                          const Tensor& A_log, const Tensor& D, Tensor& state, const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H,
@@ -739,7 +844,7 @@ Tensor Kernels::ssm_gate_norm(const Tensor& y, const Tensor& proj, int64_t z_col
 }
 
 // ------------------------------------------------------------------------------ mixture of experts
-Kernels::MoePlan Kernels::moe_route(const Tensor& h, const Tensor& router, int top, float weight_eps, int tile_rows) {
+Kernels::MoePlan Kernels::moe_route(const Tensor& h, const Tensor& router, int top, float weight_eps, int tile_rows, const Tensor* bias) {
   expect(h, "router input", dtype_);
   expect(router, "router weight", dtype_);
   if (h.shape.size() != 2 || router.shape.size() != 2 || router.dim(1) != h.dim(1) || top < 1 || top > router.dim(0))
@@ -759,7 +864,13 @@ Kernels::MoePlan Kernels::moe_route(const Tensor& h, const Tensor& router, int t
   p.tile_expert = empty({tiles}, DType::I32);
   p.expert_start = empty({E + 1}, DType::I32);
   Tensor logits = empty({T, E}, DType::F32);
-  call(fn_->moe_route(p.idx.data, p.wts.data, logits.data, h.data, router.data, (int)T, (int)h.dim(1), (int)E, top, weight_eps, stream));
+  if (bias) {
+    const int bf = norm_weight(*bias, "router bias", E);
+    call(fn_->moe_route_bias(p.idx.data, p.wts.data, logits.data, h.data, router.data, bias->data, bf, (int)T, (int)h.dim(1), (int)E, top, weight_eps,
+                             stream));
+  } else {
+    call(fn_->moe_route(p.idx.data, p.wts.data, logits.data, h.data, router.data, (int)T, (int)h.dim(1), (int)E, top, weight_eps, stream));
+  }
   call(fn_->moe_plan(p.idx.data, p.row_pair.data, p.row_token.data, p.pair_row.data, p.tile_expert.data, p.expert_start.data, (int)T, top, (int)E,
                      tile_rows, stream));
   return p;
@@ -791,11 +902,38 @@ Tensor Kernels::moe_down(const Tensor& act, const Tensor& w_down, const MoePlan&
   return y;
 }
 
-Tensor Kernels::moe_sum(const Tensor& y, const MoePlan& plan) {
+Tensor Kernels::moe_up_plain(const Tensor& h, const Tensor& w, const MoePlan& plan) {
+  expect(h, "experts' input", dtype_);
+  expect(w, "experts' weights", dtype_);
+  if (h.shape.size() != 2 || w.shape.size() != 3 || w.dim(0) != plan.experts || w.dim(2) != h.dim(1) || plan.idx.dim(0) != h.dim(0) ||
+      plan.tile_rows != 16)
+    throw EngineError("experts (up): input " + h.describe() + ", weights " + w.describe());
+  const int64_t T = h.dim(0), N = w.dim(1);
+  Tensor act = empty({plan.row_pair.dim(0), N});
+  call(fn_->moe_up_plain(act.data, N, h.data, h.dim(1), w.data, plan.row_pair.data, plan.row_token.data, plan.tile_expert.data, (int)T, plan.top,
+                         plan.experts, (int)N, (int)h.dim(1), stream));
+  return act;
+}
+
+Tensor Kernels::moe_glu(const Tensor& gate_up, float limit, float slope, float shift) {
+  expect(gate_up, "gate and up outputs", dtype_);
+  if (gate_up.shape.size() != 2 || gate_up.dim(1) % 2) throw EngineError("gated activation: rows are " + gate_up.describe());
+  const int64_t F = gate_up.dim(1) / 2;
+  Tensor out = empty({gate_up.dim(0), F});
+  call(fn_->moe_glu(out.data, gate_up.data, gate_up.dim(0), (int)F, limit, slope, shift, stream));
+  return out;
+}
+
+Tensor Kernels::moe_sum(const Tensor& y, const MoePlan& plan, const Tensor* extra) {
   expect(y, "experts' outputs", dtype_);
   if (y.shape.size() != 2 || y.dim(0) != plan.row_pair.dim(0)) throw EngineError("experts (sum): outputs " + y.describe());
   const int64_t T = plan.idx.dim(0), W = y.dim(1);
   Tensor out = empty({T, W}, DType::F32);
+  if (extra) {
+    expect(*extra, "the shared expert's output", dtype_, {T, W});
+    call(fn_->moe_combine_add(out.data, y.data, plan.wts.data, plan.pair_row.data, extra->data, (int)T, (int)W, plan.top, stream));
+    return out;
+  }
   call(fn_->moe_combine(out.data, y.data, plan.wts.data, plan.pair_row.data, (int)T, (int)W, plan.top, stream));
   return out;
 }

@@ -179,6 +179,23 @@ class Kernels {
   // cosine and sine times mag; no head norms.
   Tensor qkv_post_angles(const Tensor& qkv, int nq, int nkv, int d, const Tensor* k_cache, const Tensor* v_cache, int page_size,
                          const Tensor& inv_freq, float mag, const Tensor& positions, const Tensor* slots);
+  // The same with head norms before the rotation: q and k heads are normed over their first norm_d elements with the
+  // weights q_w and k_w [norm_d] (either may be null) and eps; elements beyond norm_d (a padded head) come out zero.  The
+  // rows of qkv may hold more columns than the heads' (what follows them is not read).
+  Tensor qkv_post_norm_angles(const Tensor& qkv, int nq, int nkv, int d, const Tensor* k_cache, const Tensor* v_cache, int page_size,
+                              const Tensor* q_w, const Tensor* k_w, int norm_d, float eps, const Tensor& inv_freq, float mag, const Tensor& positions,
+                              const Tensor* slots);
+  // x [T, W] <- x * act(gate[:, gate_col : gate_col + W]); kind 0: the logistic function, 1: z * logistic(z).
+  void gate_mul(Tensor& x, const Tensor& gate, int64_t gate_col, int kind);
+  // ---- gated linear attention with a decay per key channel (delta.hip)
+  // sigmoid(a + bias)^(1 / root) as floats [T, H, d]; a: elements [T, H d].
+  Tensor gla_decay(const Tensor& a, const Tensor& bias, int H, int d, float root);
+  // S <- diag(g) S + k v^T, o = S^T (q * q_scale) per head and token; x: element rows with q, k (H heads of d) and v (H
+  // heads of dv) at the three columns.  Returns o [T, H, dv] floats; the state [slots, >= H d dv] moves on.
+  Tensor gla_rule(const Tensor& x, int64_t q_col, int64_t k_col, int64_t v_col, const Tensor& decay, Tensor& state, const Tensor& cu_q,
+                  const Tensor& positions, const Tensor& slots, int H, int d, int dv, float q_scale);
+  // delta_out with the gate at columns [gate_col, gate_col + H dv) of a wider tensor and a choice of its activation.
+  Tensor gated_head_norm(const Tensor& o, const Tensor& gate, int64_t gate_col, const Tensor& w, int H, int dv, float eps, int gate_kind, int64_t width);
   // ---- a state-space recurrence with one decay per head (ssm.hip)
   // xbc: floats [T, C] with x (H heads of P) from column 0, B (G groups of N) from b_col, C from c_col; dt: head h's step
   // size before its activation at column dt_col + h of proj (elements).  Returns y [T, H, P] floats; the state moves on.
@@ -195,13 +212,18 @@ class Kernels {
     int top = 0, experts = 0, tile_rows = 16;   // an expert's rows are padded to whole tiles of this many
   };
   // tile_rows 16: for moe_up / moe_down; 128: for gemm_grouped, whose blocks are the plan's tiles.
-  MoePlan moe_route(const Tensor& h, const Tensor& router, int top, float weight_eps, int tile_rows = 16);
+  // bias: [experts], added to the logits before the choice, or null.
+  MoePlan moe_route(const Tensor& h, const Tensor& router, int top, float weight_eps, int tile_rows = 16, const Tensor* bias = nullptr);
+  // h W^T of every (token, choice) in the plan's rows, no activation; w [E, N, width]; result [rows, N] elements.
+  Tensor moe_up_plain(const Tensor& h, const Tensor& w, const MoePlan& plan);
+  // The gated activation of rows [gate: F | up: F]: min(gate, limit) * sigmoid(slope * .) * (clamp(up, +-limit) + shift), [rows, F].
+  Tensor moe_glu(const Tensor& gate_up, float limit, float slope, float shift);
   // relu(h W_up^T)^2 of every (token, choice) in the plan's rows; w_up [E, ff, width]; result [rows, ff] elements.
   Tensor moe_up(const Tensor& h, const Tensor& w_up, const MoePlan& plan);
   // The chosen experts' down projections of the plan's rows, [rows, width] elements; w_down [E, width, ff].
   Tensor moe_down(const Tensor& act, const Tensor& w_down, const MoePlan& plan);
   // The weighted sum of a token's rows, floats [T, width].
-  Tensor moe_sum(const Tensor& y, const MoePlan& plan);
+  Tensor moe_sum(const Tensor& y, const MoePlan& plan, const Tensor* extra = nullptr);   // extra [T, width] elements: added last
   // act [M, K] in blocks of 128 rows, block b times the matrix block_weights[b] of w [matrices, N, K] (negative: the
   // block is skipped); [M, N] elements, the bits gemm gives for the same rows and matrix.  K in whole pairs of slabs.
   Tensor gemm_grouped(const Tensor& act, const Tensor& w, const Tensor& block_weights);

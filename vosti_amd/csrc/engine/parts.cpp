@@ -373,7 +373,8 @@ struct AttentionItems {
 // denominator), exact_weights (the probabilities meet the values in 32-bit), own_kv 0 (the layer has no key and
 // value projections: it always reads another execution's cache), block (positions are cut into blocks of this many from
 // the sequence's start, and a query sees the earlier keys of its own block only; sink 2 is the constant 0 as every
-// head's sink).  The cache and the kernels see one head size: the
+// head's sink), output_gate (the heads' outputs are multiplied element by element with sigmoid(W_gate h), a projection of
+// the mixer's own input, before the output projection).  The cache and the kernels see one head size: the
 // larger of the two, rounded up to 16; the shorter of keys and values is padded with zeros in the weights, so that
 // the projections write the padding and the output projection ignores it.
 class Attention : public Mixer {
@@ -383,7 +384,7 @@ class Attention : public Mixer {
         dk_((int)s.integer("head_dim")), dv_((int)s.integer("value_dim", s.integer("head_dim"))), scale_((float)s.number("scale")),
         window_((int)s.integer("window", 0)), keep_((int)s.integer("keep_first", 0)), softcap_((float)s.number("softcap", 0.0)),
         bias_(s.integer("bias", 0) != 0), sink_((int)s.integer("sink", 0)), exact_(s.integer("exact_weights", 0) != 0),
-        own_kv_(s.integer("own_kv", 1) != 0), block_((int)s.integer("block", 0)) {
+        own_kv_(s.integer("own_kv", 1) != 0), block_((int)s.integer("block", 0)), gate_(s.integer("output_gate", 0) != 0) {
     d_ = (int)round_up(std::max(dk_, dv_), 16);
     if (nq_ % nkv_) throw ConfigError(std::to_string(nq_) + " heads are not a multiple of " + std::to_string(nkv_) + " kv heads");
     if (dk_ < 1 || dv_ < 1 || d_ > 256)
@@ -394,8 +395,8 @@ class Attention : public Mixer {
     if (const PartSpec* p = s.part("q_norm")) q_norm_ = build_part<Norm>("norm", *p, k);
     if (const PartSpec* p = s.part("k_norm")) k_norm_ = build_part<Norm>("norm", *p, k);
     if (const PartSpec* p = s.part("position")) position_ = build_part<PositionEncoding>("position", *p, k);
-    if ((bias_ && (q_norm_ || k_norm_ || position_)) || (d_ != dk_ && (q_norm_ || k_norm_)))
-      throw ConfigError("attention: biases are not built together with head norms or a position encoding, nor padded head sizes with head norms");
+    if (bias_ && (q_norm_ || k_norm_ || position_))
+      throw ConfigError("attention: biases are not built together with head norms or a position encoding");
   }
   // The kernel with capped scores serves every one of these.
   bool capped() const { return softcap_ > 0.f || keep_ > 0 || sink_ || exact_ || block_ > 0; }
@@ -416,6 +417,7 @@ class Attention : public Mixer {
       ParamDecl sinks{"sinks", {(int64_t)nq_}, true, true, -1.0, 1.0};
       p.push_back(sinks);
     }
+    if (gate_) p.push_back({"gate_proj.weight", {(int64_t)nq_ * dv_, hidden_}});
     return p;
   }
   std::vector<std::pair<std::string, Part*>> children() override {
@@ -433,6 +435,8 @@ class Attention : public Mixer {
       rows.push_back(pad_row_blocks(need(t, "k_proj.weight"), nkv_, dk_, d_));
       rows.push_back(pad_row_blocks(need(t, "v_proj.weight"), nkv_, dv_, d_));
     }
+    // The output gate's rows follow the heads', so that the steps between the projections read the heads where they were.
+    if (gate_) rows.push_back(pad_row_blocks(need(t, "gate_proj.weight"), nq_, dv_, d_));
     w_qkv_ = rows.size() > 1 ? stack_rows(rows) : rows[0];
     w_o_ = pad_column_blocks(need(t, "o_proj.weight"), nq_, dv_, d_);
     if (bias_) {
@@ -501,7 +505,7 @@ class Attention : public Mixer {
   }
   // Workspace with which the two projections of T rows take their faster route, where there is one.
   int64_t gemm_floats(int64_t T) const {
-    return std::max(kernels.gemm_workspace_floats(T, (int64_t)(nq_ + 2 * nkv_) * d_, hidden_),
+    return std::max(kernels.gemm_workspace_floats(T, (int64_t)(nq_ + 2 * nkv_ + (gate_ ? nq_ : 0)) * d_, hidden_),
                     kernels.gemm_workspace_floats(T, hidden_, (int64_t)nq_ * d_));
   }
   int64_t workspace_floats(HostStep& step) override {
@@ -526,9 +530,25 @@ class Attention : public Mixer {
     if (gf) ws_t = ctx.workspace(gf);
     const Tensor* ws = gf ? &ws_t : nullptr;
     if (cache.writable && !own_kv_) throw EngineError("an attention layer without key and value projections was given a cache to write");
-    const Tensor qkv = k.gemm(x, cache.writable ? w_qkv_ : w_qkv_.rows(0, (int64_t)nq_ * d_), ws);
+    // Rows of the stacked weight: q, then k and v (where the layer has them), then the output gate.  An execution that
+    // reads another's cache projects q and the gate alone; without a gate, q's rows are the first of the weight.
+    const int64_t heads_w = (int64_t)(nq_ + (cache.writable ? 2 * nkv_ : 0)) * d_;
+    Tensor qkv_all;
+    if (cache.writable || !own_kv_) qkv_all = k.gemm(x, w_qkv_, ws);
+    else if (!gate_) qkv_all = k.gemm(x, w_qkv_.rows(0, (int64_t)nq_ * d_), ws);
+    else throw EngineError("an attention layer with an output gate and projections of its own cannot read another execution's cache");
+    const bool padded_norm = d_ != dk_ && (q_norm_ || k_norm_);
+    const bool norm_angles = position_ && position_->angle_frequencies() && (q_norm_ || k_norm_) && fused();
+    if (padded_norm && !norm_angles) throw ConfigError("attention: head norms on padded head sizes are built for rotations by computed angles only");
+    // The kernels between the projections take rows of exactly the heads' width, except the one that says otherwise.
+    const Tensor qkv = (qkv_all.dim(1) == heads_w || norm_angles) ? qkv_all : k.columns(qkv_all, 0, heads_w);
     Tensor q;
-    if (bias_) {
+    if (norm_angles) {
+      const Norm* en = q_norm_ ? q_norm_.get() : k_norm_.get();
+      q = k.qkv_post_norm_angles(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size,
+                                 q_norm_ ? q_norm_->row_scale_weight() : nullptr, k_norm_ && cache.writable ? k_norm_->row_scale_weight() : nullptr, dk_,
+                                 en->eps(), *position_->angle_frequencies(), position_->magnitude(), ctx.positions, &tables.slots);
+    } else if (bias_) {
       const int64_t bw = (int64_t)(nq_ + (cache.writable ? 2 * nkv_ : 0)) * d_;
       q = k.qkv_post_bias(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size, &tables.slots, b_qkv_.rows(0, bw));
     } else if (position_ && position_->angle_frequencies() && !q_norm_ && !k_norm_) {
@@ -565,7 +585,9 @@ class Attention : public Mixer {
         k.paged_attention(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, decode_items, 1, scale_, window_,
                           m.decode_bound, m.nseg, &scratch);
     }
-    return k.gemm(out.view({T, (int64_t)nq_ * d_}), w_o_, ws);
+    Tensor heads = out.view({T, (int64_t)nq_ * d_});
+    if (gate_) k.gate_mul(heads, qkv_all, heads_w, 0);
+    return k.gemm(heads, w_o_, ws);
   }
 
  private:
@@ -598,6 +620,7 @@ class Attention : public Mixer {
   int sink_;                          // 0: none, 1: a learned number per head, 2: the constant 0
   bool exact_, own_kv_;
   int block_;                         // > 0: a row sees the keys of its own block of this many positions only
+  bool gate_;                         // the heads' outputs times sigmoid(W_gate h)
   std::unique_ptr<Norm> q_norm_, k_norm_;
   std::unique_ptr<PositionEncoding> position_;
   Tensor w_qkv_, w_o_, b_qkv_, sinks_;
@@ -804,6 +827,76 @@ class ChannelDelta : public Mixer {
   Tensor w_in_, w_decay_up_, w_gate_up_, conv_, A_log_, dt_bias_, out_norm_, w_o_;
 };
 
+// Gated linear attention with one decay per head and key channel.  For the mixer's input h:
+//   q = W_q h * key size^(-1/2), k = W_k h (heads x key size), v = W_v h (heads x value size);
+//   g = sigmoid(W_a2 (W_a1 h) + b_a2)^(1 / decay_root) per head and key channel;
+//   per head, token by token:  S <- diag(g) S + k v^T;  o = S^T q;
+//   y = o / sqrt(mean(o^2) + eps) * w_norm * silu(W_g h) per head; out = W_o y.
+// A request's state slot holds the heads' S in 32-bit, zero at the request's start.  The five input projections are one
+// launch (their weights stacked, each section padded to a multiple of 8 rows with zero rows, so that the decay's second
+// projection reads its columns in place); decays, recurrence and read-out are kernels of delta.hip, all in 32-bit: the
+// recurrence is the delta rule's walk without its correction term.
+class GatedLinearAttention : public Mixer {
+ public:
+  GatedLinearAttention(const PartSpec& s, Kernels& k)
+      : Mixer(k), hidden_(s.integer("hidden_size")), H_((int)s.integer("num_heads")), d_((int)s.integer("key_dim")), dv_((int)s.integer("value_dim")),
+        decay_rank_(s.integer("decay_rank", 0)), root_((float)s.number("decay_root", 1.0)), eps_((float)s.number("eps")) {
+    if (H_ < 1 || d_ < 1 || dv_ < 1 || d_ > 1024) throw ConfigError("linear attention: heads of " + std::to_string(d_) + " x " + std::to_string(dv_));
+    if (!(root_ > 0.f)) throw ConfigError("linear attention: 'decay_root' must be positive");
+    qk_ = round_up((int64_t)H_ * d_, 8);
+    v_ = round_up((int64_t)H_ * dv_, 8);
+  }
+  std::vector<ParamDecl> params() const override {
+    const int64_t hd = (int64_t)H_ * d_, hv = (int64_t)H_ * dv_;
+    const int64_t ra = decay_rank_ > 0 ? decay_rank_ : -1;      // 0: the rank is whatever the stored tensors have
+    ParamDecl q{"q_proj.weight", {hd, hidden_}}, kk{"k_proj.weight", {hd, hidden_}}, vv{"v_proj.weight", {hv, hidden_}};
+    q.p0 = kk.p0 = vv.p0 = 0.1;
+    ParamDecl a1{"decay_down.weight", {ra, hidden_}}, a2{"decay_up.weight", {hd, ra}};
+    a1.free_size = a2.free_size = std::max<int64_t>(8, hidden_ / 16);
+    a2.p0 = 0.5;
+    ParamDecl bias{"decay_up.bias", {hd}, true, true, 1.0, 5.0}, norm{"out_norm.weight", {(int64_t)dv_}, true, true, 0.9, 1.1};
+    return {q, kk, vv, {"gate_proj.weight", {hv, hidden_}}, a1, a2, bias, norm, {"o_proj.weight", {hidden_, hv}}};
+  }
+  void load(std::map<std::string, Tensor>& t) override {
+    const Tensor a1 = need(t, "decay_down.weight"), a2 = need(t, "decay_up.weight");
+    if (a1.dim(0) != a2.dim(1)) throw EngineError("linear attention: the decay's two projections do not fit each other: " + a1.describe() + " with " + a2.describe());
+    const int64_t ra = round_up(a1.dim(0), 8);
+    w_in_ = stack_rows({pad_matrix(need(t, "q_proj.weight"), qk_, hidden_), pad_matrix(need(t, "k_proj.weight"), qk_, hidden_),
+                        pad_matrix(need(t, "v_proj.weight"), v_, hidden_), pad_matrix(need(t, "gate_proj.weight"), v_, hidden_),
+                        pad_matrix(a1, ra, hidden_)});
+    gate_col_ = 2 * qk_ + v_;
+    decay_col_ = gate_col_ + v_;
+    w_decay_up_ = pad_matrix(a2, a2.dim(0), ra);
+    decay_bias_ = need(t, "decay_up.bias");
+    out_norm_ = need(t, "out_norm.weight");
+    w_o_ = pad_matrix(need(t, "o_proj.weight"), hidden_, v_);      // the read-out's width as whole 16-byte vectors
+  }
+  CacheNeed cache_need() const override {
+    CacheNeed n;
+    n.kind = CacheNeed::State;
+    n.state_shape = {(int64_t)H_ * d_ * dv_};
+    n.state_dtype = DType::F32;
+    return n;
+  }
+  Tensor forward(const Tensor& x, StepContext& ctx, CacheEntry& cache) override {
+    if (cache.kind != CacheNeed::State) throw EngineError("linear attention was handed a cache entry without state");
+    Kernels& k = kernels;
+    const Tensor proj = k.gemm(x, w_in_);
+    const Tensor decay = k.gla_decay(k.gemm_columns(proj, decay_col_, w_decay_up_), decay_bias_, H_, d_, root_);
+    const Tensor o = k.gla_rule(proj, 0, qk_, 2 * qk_, decay, cache.state, ctx.cu_q, ctx.positions, ctx.state_slots, H_, d_, dv_,
+                                1.f / std::sqrt((float)d_));
+    return k.gemm(k.gated_head_norm(o, proj, gate_col_, out_norm_, H_, dv_, eps_, 1, v_), w_o_);
+  }
+
+ private:
+  int64_t hidden_;
+  int H_, d_, dv_;
+  int64_t decay_rank_;
+  float root_, eps_;
+  int64_t qk_ = 0, v_ = 0, gate_col_ = 0, decay_col_ = 0;
+  Tensor w_in_, w_decay_up_, decay_bias_, out_norm_, w_o_;
+};
+
 // A layer without a feed-forward names this kind; an arrangement that allows it never calls it.
 class NoFeedForward : public FeedForward {
  public:
@@ -811,7 +904,8 @@ class NoFeedForward : public FeedForward {
   Tensor forward(const Tensor&, StepContext&) override { throw EngineError("a layer without a feed-forward was asked to run one"); }
 };
 
-// A residual stream x in 32-bit, a norm before and after each sublayer, and a weighted sum over the stream's earlier
+// A residual stream x in 32-bit, a norm before and after each sublayer, and (kind "sandwich_depth"; kind "sandwich" ends
+// after the two sublayers, and needs the numbers residual_mult and hidden_size alone) a weighted sum over the stream's earlier
 // states at the layer's end:
 //   x <- x + m * norm_mixer_out(mixer(norm_mixer_in(x)));  x <- x + m * norm_ffn_out(ffn(norm_ffn_in(x))) (if the
 //   layer has a feed-forward);  X_(i+1) = x;  passed on: sum over j <= i + 1 of depth_weights[j] * X_j,
@@ -828,8 +922,9 @@ class SandwichDepthBlock : public Block {
       return it->second;
     };
     mult_ = (float)number("residual_mult");
-    depth_ = (int)number("depth");
-    states_ = (int)number("states");
+    deep_ = numbers.count("states") > 0;
+    depth_ = deep_ ? (int)number("depth") : 0;
+    states_ = deep_ ? (int)number("states") : 2;
     hidden_ = (int64_t)number("hidden_size");
     if (depth_ < 0 || depth_ + 1 >= states_) throw ConfigError("a sandwich_depth block at depth " + std::to_string(depth_) + " of " + std::to_string(states_) + " states");
     has_ffn_ = dynamic_cast<NoFeedForward*>(ffn_.get()) == nullptr;
@@ -839,10 +934,13 @@ class SandwichDepthBlock : public Block {
       throw ConfigError("a sandwich_depth block with a feed-forward needs the norms 'ffn_in' and 'ffn_out'");
   }
   std::vector<ParamDecl> params() const override {
+    if (!deep_) return {};
     ParamDecl w{"depth_weights", {(int64_t)depth_ + 2}, true, true, 0.0, 2.0 / (depth_ + 2)};
     return {w};
   }
-  void load(std::map<std::string, Tensor>& t) override { weights_ = need(t, "depth_weights"); }
+  void load(std::map<std::string, Tensor>& t) override {
+    if (deep_) weights_ = need(t, "depth_weights");
+  }
   std::vector<std::pair<std::string, Part*>> children() override {
     std::vector<std::pair<std::string, Part*>> c = {{"mixer", mixer_.get()}, {"feed_forward", ffn_.get()}};
     for (auto& n : norms_) c.emplace_back("norms." + n.first, n.second.get());
@@ -854,6 +952,17 @@ class SandwichDepthBlock : public Block {
     if (hidden.dtype != DType::F32 || hidden.shape.size() != 2 || hidden.dim(1) != hidden_)
       throw EngineError("a sandwich_depth block takes the 32-bit residual stream, not " + hidden.describe());
     const int64_t T = hidden.dim(0);
+    if (!deep_) {
+      // The plain arrangement (kind "sandwich"): the stream itself is passed on.
+      Tensor stream = hidden;
+      const Tensor mixed = mixer_->forward(norms_["mixer_in"]->forward(hidden), ctx, cache);
+      norms_["mixer_out"]->forward_scaled_add(mixed, hidden, stream, mult_);
+      if (has_ffn_) {
+        const Tensor fed = ffn_->forward(norms_["ffn_in"]->forward(stream), ctx);
+        norms_["ffn_out"]->forward_scaled_add(fed, stream, stream, mult_);
+      }
+      return {stream, residual};
+    }
     Tensor& states = ctx.carry["stream.states"];
     if (depth_ == 0) {
       states = k.empty({(int64_t)states_, T, hidden_}, DType::F32);
@@ -880,7 +989,7 @@ class SandwichDepthBlock : public Block {
   float mult_ = 1.f;
   int depth_ = 0, states_ = 0;
   int64_t hidden_ = 0;
-  bool has_ffn_ = true;
+  bool has_ffn_ = true, deep_ = true;    // deep_: the weighted sum over earlier states ends the layer
   Tensor weights_;
 };
 
@@ -1017,19 +1126,40 @@ class PairMean : public Mixer {
 // sum plus weight_eps; the output is the weighted sum of the chosen experts' outputs, in 32-bit.  The experts' weights
 // lie stacked, [experts, ff, width] and [experts, width, ff] (ff padded to a multiple of 64 with zeros), and the two
 // projections run as grouped products over the (token, choice) pairs sorted by expert (moe.hip, gemm.hip).
+//
+// Further numbers, all optional: router_bias (a bias per expert on the logits, which choice and weights both see; with
+// weight_eps 0 the weights are then the softmax over the chosen logits alone), gated (an expert is
+// W_down (g * sigmoid(glu_slope * g) * (u + up_shift)) with g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit)),
+// shared_size (> 0: one more expert of that inner size and the same form, with shared_limit, that every token uses
+// with weight 1; its output is added to the sum).
 class RoutedExperts : public FeedForward {
  public:
   RoutedExperts(const PartSpec& s, Kernels& k)
       : FeedForward(k), hidden_(s.integer("hidden_size")), inter_(s.integer("intermediate_size")), experts_((int)s.integer("experts")),
-        top_((int)s.integer("top")), weight_eps_((float)s.number("weight_eps", 0.0)) {
+        top_((int)s.integer("top")), weight_eps_((float)s.number("weight_eps", 0.0)), bias_(s.integer("router_bias", 0) != 0),
+        gated_(s.integer("gated", 0) != 0), limit_((float)s.number("limit", 0.0)), slope_((float)s.number("glu_slope", 1.0)),
+        shift_((float)s.number("up_shift", 0.0)), shared_(s.integer("shared_size", 0)), shared_limit_((float)s.number("shared_limit", 0.0)) {
     if (experts_ < 1 || top_ < 1 || top_ > experts_) throw ConfigError("a mixture of " + std::to_string(experts_) + " experts cannot choose " + std::to_string(top_));
+    if (gated_ && !(limit_ > 0.f)) throw ConfigError("gated experts need a positive 'limit'");
+    if (shared_ < 0 || (shared_ > 0 && (!gated_ || !(shared_limit_ > 0.f))))
+      throw ConfigError("a shared expert is built in the gated form, with a positive 'shared_limit'");
   }
   std::vector<ParamDecl> params() const override {
     std::vector<ParamDecl> p = {{"router.weight", {(int64_t)experts_, hidden_}}};
     p[0].p0 = 0.1;
+    if (bias_) {
+      ParamDecl b{"router.bias", {(int64_t)experts_}, true, true, -0.5, 0.5};
+      p.push_back(b);
+    }
     for (int e = 0; e < experts_; ++e) {
+      if (gated_) p.push_back({"experts." + std::to_string(e) + ".gate_proj.weight", {inter_, hidden_}});
       p.push_back({"experts." + std::to_string(e) + ".up_proj.weight", {inter_, hidden_}});
       p.push_back({"experts." + std::to_string(e) + ".down_proj.weight", {hidden_, inter_}});
+    }
+    if (shared_ > 0) {
+      p.push_back({"shared.gate_proj.weight", {shared_, hidden_}});
+      p.push_back({"shared.up_proj.weight", {shared_, hidden_}});
+      p.push_back({"shared.down_proj.weight", {hidden_, shared_}});
     }
     return p;
   }
@@ -1037,28 +1167,42 @@ class RoutedExperts : public FeedForward {
     router_ = need(t, "router.weight");
     const int64_t padded = round_up(inter_, 64);              // whole pairs of slabs, so that the tile product takes it
     std::vector<Tensor> up, down;
+    if (bias_) router_bias_ = need(t, "router.bias");
+    if (shared_ > 0) {
+      const int64_t sp = round_up(shared_, 64);
+      w_shared_in_ = stack_rows({pad_matrix(need(t, "shared.gate_proj.weight"), sp, hidden_), pad_matrix(need(t, "shared.up_proj.weight"), sp, hidden_)});
+      w_shared_down_ = pad_matrix(need(t, "shared.down_proj.weight"), hidden_, sp);
+    }
     for (int e = 0; e < experts_; ++e) {
+      // A gated expert's first product gives the gate's outputs and then the up projection's, each padded alike.
+      if (gated_) up.push_back(pad_matrix(need(t, "experts." + std::to_string(e) + ".gate_proj.weight"), padded, hidden_));
       up.push_back(pad_matrix(need(t, "experts." + std::to_string(e) + ".up_proj.weight"), padded, hidden_));
       Tensor d = pad_matrix(need(t, "experts." + std::to_string(e) + ".down_proj.weight"), hidden_, padded);
       down.push_back(d.view({hidden_ * padded / 8, 8}));     // stacked as rows of one width whatever the matrices' own
     }
-    w_up_ = stack_rows(up).view({(int64_t)experts_, padded, hidden_});
+    w_up_ = stack_rows(up).view({(int64_t)experts_, (gated_ ? 2 : 1) * padded, hidden_});
     w_down_ = stack_rows(down).view({(int64_t)experts_, hidden_, padded});
   }
   Tensor forward(const Tensor& x, StepContext&) override {
     Kernels& k = kernels;
     const int64_t pairs = x.dim(0) * top_;
+    const Tensor* bias = bias_ ? &router_bias_ : nullptr;
+    Tensor shared;
+    if (shared_ > 0) shared = k.gemm(k.moe_glu(k.gemm(x, w_shared_in_), shared_limit_, slope_, shift_), w_shared_down_);
+    const Tensor* extra = shared_ > 0 ? &shared : nullptr;
     // Few rows an expert: products over tiles of 16 rows that stream an expert's weights once a tile.  Many (prompts):
     // the rows are sorted by expert into blocks of 128 and go through the engine's tile product, every block with its
     // expert's matrix.  Both are launched from numbers on the GPU alone and give the same bits.
-    if (pairs < (int64_t)kRowsAnExpertForTiles * experts_ || !k.gemm_grouped_takes(hidden_) || !k.gemm_grouped_takes(w_up_.dim(1))) {
-      const Kernels::MoePlan plan = k.moe_route(x, router_, top_, weight_eps_);
-      return k.moe_sum(k.moe_down(k.moe_up(x, w_up_, plan), w_down_, plan), plan);
+    if (pairs < (int64_t)kRowsAnExpertForTiles * experts_ || !k.gemm_grouped_takes(hidden_) || !k.gemm_grouped_takes(w_down_.dim(2))) {
+      const Kernels::MoePlan plan = k.moe_route(x, router_, top_, weight_eps_, 16, bias);
+      const Tensor act = gated_ ? k.moe_glu(k.moe_up_plain(x, w_up_, plan), limit_, slope_, shift_) : k.moe_up(x, w_up_, plan);
+      return k.moe_sum(k.moe_down(act, w_down_, plan), plan, extra);
     }
-    const Kernels::MoePlan plan = k.moe_route(x, router_, top_, weight_eps_, 128);
+    const Kernels::MoePlan plan = k.moe_route(x, router_, top_, weight_eps_, 128, bias);
     Tensor act = k.gemm_grouped(k.gather_rows(x, plan.row_token), w_up_, plan.tile_expert);
-    k.relu_square(act);
-    return k.moe_sum(k.gemm_grouped(act, w_down_, plan.tile_expert), plan);
+    if (gated_) act = k.moe_glu(act, limit_, slope_, shift_);
+    else k.relu_square(act);
+    return k.moe_sum(k.gemm_grouped(act, w_down_, plan.tile_expert), plan, extra);
   }
   static constexpr int kRowsAnExpertForTiles = 32;
 
@@ -1066,7 +1210,11 @@ class RoutedExperts : public FeedForward {
   int64_t hidden_, inter_;
   int experts_, top_;
   float weight_eps_;
-  Tensor router_, w_up_, w_down_;
+  bool bias_, gated_;
+  float limit_, slope_, shift_;
+  int64_t shared_;
+  float shared_limit_;
+  Tensor router_, router_bias_, w_up_, w_down_, w_shared_in_, w_shared_down_;
 };
 
 // Mixer and feed-forward side by side on a residual stream x in 32-bit: x <- x + (mixer(norm_mixer_in(x)) +
@@ -1129,6 +1277,14 @@ void register_standard_parts() {
                                         std::map<std::string, std::unique_ptr<Norm>> n, const std::map<std::string, double>& numbers) {
       return std::unique_ptr<Block>(new SandwichDepthBlock(k, std::move(m), std::move(f), std::move(n), numbers));
     });
+    register_block("sandwich", [](Kernels& k, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
+                                  std::map<std::string, std::unique_ptr<Norm>> n, const std::map<std::string, double>& numbers) {
+      std::map<std::string, double> plain = numbers;
+      plain.erase("states");
+      plain.erase("depth");
+      return std::unique_ptr<Block>(new SandwichDepthBlock(k, std::move(m), std::move(f), std::move(n), plain));
+    });
+    register_part("mixer", "gated_linear_attention", factory<GatedLinearAttention>());
     register_part("embedding", "token_embedding_scaled", factory<ScaledEmbedding>());
     register_part("position", "rotary_stretched", factory<RotaryStretched>());
     register_part("mixer", "state_space", factory<StateSpace>());

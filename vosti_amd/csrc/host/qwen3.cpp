@@ -8,6 +8,7 @@
 #include <cmath>
 
 #include "qwen3.h"
+#include "pabavik.h"
 #include "povatar.h"
 #include "tezinex.h"
 
@@ -192,6 +193,7 @@ void register_builtin_architectures() {
   register_architecture("Qwen3ForCausalLM", "qwen3", [](const Json& raw) { return qwen3_model_spec(qwen3_config(raw)); });
   register_architecture("Tezinex", "tezinex", tezinex_model_spec);
   register_architecture("Povatar", "povatar", povatar_model_spec);
+  register_architecture("Pabavik", "pabavik", pabavik_model_spec);
 }
 
 }  // namespace vosti

@@ -23,8 +23,9 @@
 // split the row's 16-byte vectors (vector v goes to wave (v / 64) % 4, lane v % 64), a lane adds its products in ascending
 // order (fused multiply-adds), a butterfly follows over the lanes and the four waves' sums are added in wave order: the
 // order depends on the width alone.
+// bias: one number an expert that is added to its logit (elements or floats), or null.
 __global__ __launch_bounds__(256) void moe_logits_kernel(float* __restrict__ z, const elem_t* __restrict__ h, const elem_t* __restrict__ router,
-                                                         int T, int W, int E) {
+                                                         int T, int W, int E, const void* __restrict__ bias, int bias_is_f32) {
   __shared__ float part[4][MOE_ROUTE_TOKENS];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int t0 = blockIdx.x * MOE_ROUTE_TOKENS, e = blockIdx.y;
@@ -55,6 +56,7 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(float* __restrict__ z, 
     v = v + part[1][threadIdx.x];
     v = v + part[2][threadIdx.x];
     v = v + part[3][threadIdx.x];
+    if (bias != nullptr) v = v + load_weight(bias, bias_is_f32, e);
     z[(int64_t)(t0 + threadIdx.x) * E + e] = v;
   }
 }
@@ -164,7 +166,9 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restric
 #define MOE_KC_SLABS (MOE_KC / VK_SLAB)
 #define MOE_WAVES 8
 #define MOE_W 4
-template <bool UP>
+// MODE 0: the rows themselves are the inputs (down); 1: the rows' tokens, with the squared-relu activation; 2: the rows'
+// tokens, the sum as it is (an activation of two products' outputs follows in a launch of its own).
+template <int MODE>
 __global__ __launch_bounds__(64 * MOE_WAVES) void moe_gemm_kernel(elem_t* __restrict__ out, int64_t ldo, const elem_t* __restrict__ x, int64_t ldx,
                                                                   const elem_t* __restrict__ w, int64_t expert_stride,
                                                                   const int32_t* __restrict__ row_pair, const int32_t* __restrict__ row_token,
@@ -178,6 +182,7 @@ __global__ __launch_bounds__(64 * MOE_WAVES) void moe_gemm_kernel(elem_t* __rest
   const int f0 = blockIdx.x * 16;
   const int row = tile * MOE_TILE + r16;
   const bool x_ok = row_pair[row] >= 0;
+  constexpr bool UP = MODE != 0;
   const elem_t* xr = x + (int64_t)(UP ? row_token[row] : row) * ldx + kq * VK_VEC;
   const bool w_ok = f0 + r16 < N;
   const elem_t* wr = w + (int64_t)e * expert_stride + (int64_t)(w_ok ? f0 + r16 : 0) * K + kq * VK_VEC;
@@ -230,7 +235,7 @@ __global__ __launch_bounds__(64 * MOE_WAVES) void moe_gemm_kernel(elem_t* __rest
     const int f = f0 + kq * 4 + i;
     if (f >= N) continue;
     float v = total[i];
-    if (UP) {
+    if (MODE == 1) {
       const float rl = fmaxf(round_to_elem(v), 0.f);
       v = rl * rl;
     }
@@ -253,13 +258,36 @@ __global__ __launch_bounds__(256) void moe_relu_square_kernel(elem_t* x, int64_t
   store_elems(x + i * VK_VEC, v);
 }
 
-// out[t, c] = sum over k < top, ascending, of wts[t, k] * y[pair_row[t * top + k], c], from zero.
+// A gated expert's activation between its two products: row r of `in` holds the gate's F outputs and, from column F on,
+// the up projection's; y = g * sigmoid(slope * g) * (u + shift) with g = min(gate, limit) and u = clamp(up, -limit, limit),
+// in 32-bit, as elements [rows, F].  A thread takes a 16-byte vector (F in whole vectors).
+__global__ __launch_bounds__(256) void moe_glu_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ in, int64_t rows, int F, float limit,
+                                                      float slope, float shift) {
+  const int per = F / VK_VEC;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * per) return;
+  const int64_t r = i / per;
+  const int c = (int)(i - r * per) * VK_VEC;
+  float g[VK_VEC], u[VK_VEC];
+  load_elems(in + r * 2 * F + c, g);
+  load_elems(in + r * 2 * F + F + c, u);
+#pragma unroll
+  for (int j = 0; j < VK_VEC; ++j) {
+    const float gc = fminf(g[j], limit), uc = fminf(fmaxf(u[j], -limit), limit);
+    g[j] = (gc / (1.f + expf(-slope * gc))) * (uc + shift);
+  }
+  store_elems(out + r * F + c, g);
+}
+
+// out[t, c] = sum over k < top, ascending, of wts[t, k] * y[pair_row[t * top + k], c], from zero; then + extra[t, c]
+// (elements, the output of an expert that every token uses) where there is one.
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ out, const elem_t* __restrict__ y, const float* __restrict__ wts,
-                                                          const int32_t* __restrict__ pair_row, int W, int top) {
+                                                          const int32_t* __restrict__ pair_row, int W, int top, const elem_t* __restrict__ extra) {
   const int t = blockIdx.x;
   for (int c = blockIdx.y * 256 + threadIdx.x; c < W; c += gridDim.y * 256) {
     float acc = 0.f;
     for (int k = 0; k < top; ++k) acc = acc + wts[(int64_t)t * top + k] * to_f32(y[(int64_t)pair_row[(int64_t)t * top + k] * W + c]);
+    if (extra != nullptr) acc = acc + to_f32(extra[(int64_t)t * W + c]);
     out[(int64_t)t * W + c] = acc;
   }
 }
@@ -273,17 +301,30 @@ int vk_moe_max_tiles(int T, int top, int E, int tile_rows) {
   return (int)((pairs + busy * (tile_rows - 1)) / tile_rows);
 }
 
-// logits: scratch [T, E] floats.
-int vk_moe_route(int32_t* idx, float* wts, float* logits, const elem_t* h, const elem_t* router, int T, int W, int E, int top, float weight_eps,
-                 hipStream_t st) {
+// logits: scratch [T, E] floats.  bias [E] (elements, or floats with bias_is_f32) or null.
+static int route_launch(int32_t* idx, float* wts, float* logits, const elem_t* h, const elem_t* router, const void* bias, int bias_is_f32, int T, int W,
+                        int E, int top, float weight_eps, hipStream_t st) {
   VK_REQUIRE(T >= 0 && W > 0 && W % VK_VEC == 0 && E > 0 && top > 0 && top <= E && E <= 4096,
              "router: bad sizes T=%d W=%d E=%d top=%d (the width in whole 16-byte vectors, at most 4096 experts)", T, W, E, top);
   VK_REQUIRE(((uintptr_t)h % 16) == 0 && ((uintptr_t)router % 16) == 0, "router: operands must be 16-byte aligned");
   if (T == 0) return 0;
-  moe_logits_kernel<<<dim3((T + MOE_ROUTE_TOKENS - 1) / MOE_ROUTE_TOKENS, E), 256, 0, st>>>(logits, h, router, T, W, E);
+  moe_logits_kernel<<<dim3((T + MOE_ROUTE_TOKENS - 1) / MOE_ROUTE_TOKENS, E), 256, 0, st>>>(logits, h, router, T, W, E, bias, bias_is_f32);
   if (vk_check_launch("router (logits)")) return 1;
   moe_choose_kernel<<<(T + 3) / 4, 256, (size_t)4 * E * sizeof(float), st>>>(idx, wts, logits, T, E, top, weight_eps);
   return vk_check_launch("router (choice)");
+}
+
+int vk_moe_route(int32_t* idx, float* wts, float* logits, const elem_t* h, const elem_t* router, int T, int W, int E, int top, float weight_eps,
+                 hipStream_t st) {
+  return route_launch(idx, wts, logits, h, router, nullptr, 0, T, W, E, top, weight_eps, st);
+}
+
+// The same with a bias an expert on the logits, which both the choice and the weights see.  With weight_eps 0 the weights
+// are the softmax over the chosen logits alone: exp(z_k) / sum over the chosen exp(z_j), whatever the others are.
+int vk_moe_route_bias(int32_t* idx, float* wts, float* logits, const elem_t* h, const elem_t* router, const void* bias, int bias_is_f32, int T, int W,
+                      int E, int top, float weight_eps, hipStream_t st) {
+  VK_REQUIRE(bias != nullptr, "router: the bias is missing");
+  return route_launch(idx, wts, logits, h, router, bias, bias_is_f32, T, W, E, top, weight_eps, st);
 }
 
 int vk_moe_plan(const int32_t* idx, int32_t* row_pair, int32_t* row_token, int32_t* pair_row, int32_t* tile_expert, int32_t* expert_start, int T,
@@ -304,9 +345,32 @@ int vk_moe_up(elem_t* act, int64_t ldo, const elem_t* x, int64_t ldx, const elem
   if (T == 0) return 0;
   const int tiles = vk_moe_max_tiles(T, top, E, MOE_TILE);
   VK_REQUIRE(tiles <= 65535, "experts (up): too many tiles for one launch");
-  moe_gemm_kernel<true><<<dim3((N + 15) / 16, tiles), 64 * MOE_WAVES, 0, st>>>(act, ldo, x, ldx, w_up, (int64_t)N * K, row_pair, row_token, tile_expert,
+  moe_gemm_kernel<1><<<dim3((N + 15) / 16, tiles), 64 * MOE_WAVES, 0, st>>>(act, ldo, x, ldx, w_up, (int64_t)N * K, row_pair, row_token, tile_expert,
                                                                                N, K);
   return vk_check_launch("experts (up)");
+}
+
+// act [max_rows, ldo] elements = x[token of row] . w[expert of row], no activation; w [E, N, K].
+int vk_moe_up_plain(elem_t* act, int64_t ldo, const elem_t* x, int64_t ldx, const elem_t* w, const int32_t* row_pair, const int32_t* row_token,
+                    const int32_t* tile_expert, int T, int top, int E, int N, int K, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && top > 0 && E > 0 && N > 0 && K > 0 && K % VK_VEC == 0 && ldx % VK_VEC == 0 && ldx >= K && ldo >= N,
+             "experts (up): bad sizes N=%d K=%d (K in whole 16-byte vectors)", N, K);
+  VK_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "experts (up): operands must be 16-byte aligned");
+  if (T == 0) return 0;
+  const int tiles = vk_moe_max_tiles(T, top, E, MOE_TILE);
+  VK_REQUIRE(tiles <= 65535, "experts (up): too many tiles for one launch");
+  moe_gemm_kernel<2><<<dim3((N + 15) / 16, tiles), 64 * MOE_WAVES, 0, st>>>(act, ldo, x, ldx, w, (int64_t)N * K, row_pair, row_token, tile_expert, N, K);
+  return vk_check_launch("experts (up)");
+}
+
+// out [rows, F] elements from in [rows, 2 F]: the gated activation with clamped inputs (moe_glu_kernel).
+int vk_moe_glu(elem_t* out, const elem_t* in, int64_t rows, int F, float limit, float slope, float shift, hipStream_t st) {
+  VK_REQUIRE(rows >= 0 && F > 0 && F % VK_VEC == 0 && limit > 0.f && ((uintptr_t)out % 16) == 0 && ((uintptr_t)in % 16) == 0,
+             "experts (gated activation): bad sizes rows=%lld F=%d (whole 16-byte vectors)", (long long)rows, F);
+  if (rows == 0) return 0;
+  const int64_t n = rows * (F / VK_VEC);
+  moe_glu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(out, in, rows, F, limit, slope, shift);
+  return vk_check_launch("experts (gated activation)");
 }
 
 // y [max_rows, N] elements = act[row] . w_down[expert of row]; w_down [E, N, K]; act rows of length lda >= K.
@@ -318,7 +382,7 @@ int vk_moe_down(elem_t* y, const elem_t* act, int64_t lda, const elem_t* w_down,
   if (T == 0) return 0;
   const int tiles = vk_moe_max_tiles(T, top, E, MOE_TILE);
   VK_REQUIRE(tiles <= 65535, "experts (down): too many tiles for one launch");
-  moe_gemm_kernel<false><<<dim3((N + 15) / 16, tiles), 64 * MOE_WAVES, 0, st>>>(y, N, act, lda, w_down, (int64_t)N * K, row_pair, nullptr, tile_expert,
+  moe_gemm_kernel<0><<<dim3((N + 15) / 16, tiles), 64 * MOE_WAVES, 0, st>>>(y, N, act, lda, w_down, (int64_t)N * K, row_pair, nullptr, tile_expert,
                                                                                 N, K);
   return vk_check_launch("experts (down)");
 }
@@ -331,12 +395,24 @@ int vk_moe_relu_square(elem_t* x, int64_t n, hipStream_t st) {
   return vk_check_launch("experts (activation)");
 }
 
-int vk_moe_combine(float* out, const elem_t* y, const float* wts, const int32_t* pair_row, int T, int W, int top, hipStream_t st) {
+static int combine_launch(float* out, const elem_t* y, const float* wts, const int32_t* pair_row, const elem_t* extra, int T, int W, int top,
+                          hipStream_t st) {
   VK_REQUIRE(T >= 0 && W > 0 && top > 0, "experts (sum): bad sizes T=%d W=%d top=%d", T, W, top);
   if (T == 0) return 0;
   const int by = std::min((W + 255) / 256, 64);
-  moe_combine_kernel<<<dim3(T, by), 256, 0, st>>>(out, y, wts, pair_row, W, top);
+  moe_combine_kernel<<<dim3(T, by), 256, 0, st>>>(out, y, wts, pair_row, W, top, extra);
   return vk_check_launch("experts (sum)");
+}
+
+int vk_moe_combine(float* out, const elem_t* y, const float* wts, const int32_t* pair_row, int T, int W, int top, hipStream_t st) {
+  return combine_launch(out, y, wts, pair_row, nullptr, T, W, top, st);
+}
+
+// The same, and extra [T, W] (elements) is added to every token's sum last.
+int vk_moe_combine_add(float* out, const elem_t* y, const float* wts, const int32_t* pair_row, const elem_t* extra, int T, int W, int top,
+                       hipStream_t st) {
+  VK_REQUIRE(extra != nullptr, "experts (sum): the output to add is missing");
+  return combine_launch(out, y, wts, pair_row, extra, T, W, top, st);
 }
 
 }  // extern "C"

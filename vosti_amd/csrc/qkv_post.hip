@@ -31,6 +31,7 @@ struct QkvPostArgs {
   const int32_t* positions;  // [T]
   const int32_t* slots;      // [T]: page * P + offset, or -1
   int w_is_f32, nq, nkv, d, P, rot_half;
+  int norm_d;             // the head norm's own size: the mean of squares divides by it, and its weight has this many entries
   float eps;
 };
 
@@ -81,11 +82,11 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a, int per_wa
     }
     if (w != nullptr) {
       const float total = wave_sum_xor(part);
-      const float rr = rsqrtf(total / (float)d + a.eps);
+      const float rr = rsqrtf(total / (float)a.norm_d + a.eps);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int c = lane + 64 * i;
-        if (c < d) xv[i] = round_to_elem((xv[i] * rr) * load_weight(w, a.w_is_f32, c));
+        if (c < d) xv[i] = c < a.norm_d ? round_to_elem((xv[i] * rr) * load_weight(w, a.w_is_f32, c)) : 0.f;
       }
     }
     const bool rotate = has_rot && kind != 2;
@@ -240,7 +241,7 @@ extern "C" {
 static int qkv_post_launch(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc, elem_t* vc, const void* q_w,
                            const void* k_w, int w_is_f32, const elem_t* cos_t, const elem_t* sin_t, int rot_half,
                            const int32_t* positions, const int32_t* slots, int T, int nq, int nkv, int d, int P, float eps,
-                           const elem_t* bias, hipStream_t st, const float* inv_freq = nullptr, float mag = 1.f) {
+                           const elem_t* bias, hipStream_t st, const float* inv_freq = nullptr, float mag = 1.f, int norm_d = 0) {
   VK_REQUIRE(T >= 0 && nq >= 0 && nkv >= 0 && nq + nkv > 0, "qkv_post: bad sizes T=%d nq=%d nkv=%d", T, nq, nkv);
   VK_REQUIRE(d > 0 && d <= 256, "qkv_post: head size %d must be in 1..256", d);
   VK_REQUIRE(row_stride >= (int64_t)(nq + 2 * nkv) * d, "qkv_post: row stride %lld too small", (long long)row_stride);
@@ -250,15 +251,18 @@ static int qkv_post_launch(const elem_t* qkv, int64_t row_stride, elem_t* q_out,
   VK_REQUIRE(cos_t == nullptr || inv_freq == nullptr, "qkv_post: tables of angles or frequencies, not both");
   VK_REQUIRE(nkv == 0 || (slots != nullptr && kc != nullptr && vc != nullptr && P > 0), "qkv_post: store needs slots and caches");
   VK_REQUIRE(nq + 2 * nkv <= 65535, "qkv_post: too many heads");
+  VK_REQUIRE(norm_d >= 0 && norm_d <= d, "qkv_post: a head norm over %d of %d elements", norm_d, d);
+  if (norm_d == 0) norm_d = d;
   if (T == 0) return 0;
   QkvPostArgs a;
   a.qkv = qkv; a.row_stride = row_stride; a.q_out = q_out; a.kc = kc; a.vc = vc; a.q_w = q_w; a.k_w = k_w;
   a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.slots = slots; a.w_is_f32 = w_is_f32; a.bias = bias;
   a.nq = nq; a.nkv = nkv; a.d = d; a.P = P; a.rot_half = rot_half; a.eps = eps; a.inv_freq = inv_freq; a.mag = mag;
+  a.norm_d = norm_d;
   // Few tokens: four waves' worth of heads per workgroup, for many workgroups; many tokens: all heads of a token.
   const int heads = nq + 2 * nkv;
   const int lph = d / VK_VEC;          // lanes per head in the kernel with 16-byte accesses
-  const bool vec = inv_freq == nullptr && (d == 64 || d == 128 || d == 256) && lph <= 64 && (cos_t == nullptr || 2 * rot_half == d) &&
+  const bool vec = inv_freq == nullptr && norm_d == d && (d == 64 || d == 128 || d == 256) && lph <= 64 && (cos_t == nullptr || 2 * rot_half == d) &&
                    row_stride % VK_VEC == 0 && ((uintptr_t)qkv % 16) == 0 && (q_out == nullptr || (uintptr_t)q_out % 16 == 0) &&
                    (kc == nullptr || (uintptr_t)kc % 16 == 0) && (bias == nullptr || (uintptr_t)bias % 16 == 0) && (cos_t == nullptr || ((uintptr_t)cos_t % 16 == 0 && (uintptr_t)sin_t % 16 == 0));
   if (vec) {
@@ -301,6 +305,18 @@ int vk_qkv_post_angles(const elem_t* qkv, int64_t row_stride, elem_t* q_out, ele
   VK_REQUIRE(inv_freq != nullptr, "qkv_post: the rotation's frequencies are missing");
   return qkv_post_launch(qkv, row_stride, q_out, kc, vc, nullptr, nullptr, 0, nullptr, nullptr, rot_half, positions, slots, T, nq, nkv, d, P, 0.f,
                          nullptr, st, inv_freq, mag);
+}
+
+// Head norms and computed angles together: q and k heads are normed over their first norm_d elements (weights q_w, k_w of
+// that many entries, either may be null; the elements beyond, padding, come out zero), then turned as vk_qkv_post_angles
+// turns them.  Rows may be longer than the heads they hold (row_stride).
+int vk_qkv_post_norm_angles(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc, elem_t* vc, const void* q_w, const void* k_w,
+                            int w_is_f32, int norm_d, float eps, const float* inv_freq, float mag, int rot_half, const int32_t* positions,
+                            const int32_t* slots, int T, int nq, int nkv, int d, int P, hipStream_t st) {
+  VK_REQUIRE(inv_freq != nullptr, "qkv_post: the rotation's frequencies are missing");
+  VK_REQUIRE(norm_d > 0 && 2 * rot_half <= norm_d, "qkv_post: a rotation of %d elements in a head norm of %d", 2 * rot_half, norm_d);
+  return qkv_post_launch(qkv, row_stride, q_out, kc, vc, q_w, k_w, w_is_f32, nullptr, nullptr, rot_half, positions, slots, T, nq, nkv, d, P, eps,
+                         nullptr, st, inv_freq, mag, norm_d);
 }
 
 }  // extern "C"

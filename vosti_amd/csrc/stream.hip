@@ -64,7 +64,8 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_norm_kernel(elem_t* __r
 }
 
 // out = base + mult * norm(y), rows of the stream; out may be base.
-__global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_kernel(float* out, const float* base_rows, const elem_t* __restrict__ y,
+template <typename Y>     // the normed rows: elements, or floats
+__global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_kernel(float* out, const float* base_rows, const Y* __restrict__ y,
                                                                          const void* __restrict__ w, int w_is_f32, int H, float eps,
                                                                          float offset, float mult) {
   __shared__ float red[4];
@@ -124,8 +125,8 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_norm_vec_kernel(elem_t*
   }
 }
 
-template <int NV>
-__global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_vec_kernel(float* out, const float* base_rows, const elem_t* __restrict__ y,
+template <int NV, typename Y>
+__global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_vec_kernel(float* out, const float* base_rows, const Y* __restrict__ y,
                                                                              const void* __restrict__ w, int w_is_f32, int H, float eps,
                                                                              float offset, float mult) {
   __shared__ float red[4];
@@ -138,7 +139,7 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_vec_kernel(flo
     const int c = threadIdx.x + j * STREAM_THREADS;
     v[j] = b[j] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (c < nvec) {
-      const elem_t* p = y + base + 4 * c;
+      const Y* p = y + base + 4 * c;
       v[j] = f32x4{to_f32(p[0]), to_f32(p[1]), to_f32(p[2]), to_f32(p[3])};
       b[j] = *reinterpret_cast<const f32x4*>(base_rows + base + 4 * c);
     }
@@ -313,19 +314,33 @@ int vk_stream_norm(elem_t* out, const void* x, int x_is_f32, const void* w, int 
   return vk_check_launch("stream norm");
 }
 
-int vk_stream_norm_add(float* out, const float* base, const elem_t* y, const void* w, int w_is_f32, int rows, int H, float eps,
-                       float offset, float mult, hipStream_t st) {
+extern "C++" {
+template <typename Y>
+static int norm_add_launch(float* out, const float* base, const Y* y, const void* w, int w_is_f32, int rows, int H, float eps, float offset, float mult,
+                           hipStream_t st) {
   VK_REQUIRE(rows >= 0 && H > 0 && eps >= 0.f, "stream norm-add: bad sizes rows=%d H=%d", rows, H);
   if (rows == 0) return 0;
   const int nv = (H / 4 + STREAM_THREADS - 1) / STREAM_THREADS;
   if (H % 4 == 0 && nv <= 8 && (uintptr_t)out % 16 == 0 && (uintptr_t)base % 16 == 0) {
-#define NORM_ADD_VEC(NV) stream_norm_add_vec_kernel<NV><<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult)
+#define NORM_ADD_VEC(NV) stream_norm_add_vec_kernel<NV, Y><<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult)
     if (nv <= 1) NORM_ADD_VEC(1); else if (nv <= 2) NORM_ADD_VEC(2); else if (nv <= 4) NORM_ADD_VEC(4); else NORM_ADD_VEC(8);
 #undef NORM_ADD_VEC
   } else {
-    stream_norm_add_kernel<<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult);
+    stream_norm_add_kernel<Y><<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult);
   }
   return vk_check_launch("stream norm-add");
+}
+}  // extern "C++"
+
+int vk_stream_norm_add(float* out, const float* base, const elem_t* y, const void* w, int w_is_f32, int rows, int H, float eps,
+                       float offset, float mult, hipStream_t st) {
+  return norm_add_launch<elem_t>(out, base, y, w, w_is_f32, rows, H, eps, offset, mult, st);
+}
+
+// The same for rows that a sublayer left in 32-bit.
+int vk_stream_norm_add_f32(float* out, const float* base, const float* y, const void* w, int w_is_f32, int rows, int H, float eps,
+                           float offset, float mult, hipStream_t st) {
+  return norm_add_launch<float>(out, base, y, w, w_is_f32, rows, H, eps, offset, mult, st);
 }
 
 int vk_stream_mix(float* out, const float* states, int64_t stride, const void* coef, int coef_is_f32, int n, int64_t numel,
