@@ -1,0 +1,350 @@
+"""The Pabavik decoder through the native engine against the plain implementation (tests/plain_pabavik.py).
+
+Every test builds its own small model.  The engine is driven through its step function (given tokens in, logits out:
+what bin/trace_run drives) and through its scheduler (``generate``).  In float32 the engine must agree with the plain
+float64 implementation to a few units of 32-bit rounding; in bfloat16 to what rounding the matrix products to 16 bits
+costs.  Two cuttings of the same tokens through the engine must agree far closer than either does with the plain
+implementation: nothing may depend on portions, batches, pages or slots."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+import plain_pabavik as plain
+from pabavik_models import CONFIGS, attention, config, gla, layer, moe, random_weights, write_model
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = {"float32": 2e-4, "bfloat16": 6e-2}      # of the logits' root mean square
+SAME = {"float32": 2e-5, "bfloat16": 2e-5}           # two cuttings of the same tokens through the engine
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for seed, (name, cfg) in enumerate(CONFIGS.items()):
+        w = random_weights(cfg, 20 + seed)
+        out[name] = (write_model(tmp_path_factory.mktemp(name), cfg, w), cfg, w)
+    return out
+
+
+def engine(folder, dtype, num_pages=24, page_size=16, max_num_seqs=4, **kw):
+    from vosti_amd.engine.native import NativeEngine
+    return NativeEngine(folder, dtype=dtype, num_pages=num_pages, page_size=page_size, max_num_seqs=max_num_seqs,
+                        enable_prefix_cache=False, graphs=kw.pop("graphs", False), **kw)
+
+
+def tokens_for(cfg, n, seed):
+    return torch.randint(0, cfg["vocab"], (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def run_cut(eng, rid, tokens, cuts, finish=True):
+    """All logits of one request fed in portions of the given sizes."""
+    rows, at = [], 0
+    for c in cuts:
+        rows.append(eng.trace_step([(rid, tokens[at:at + c], list(range(c)))]))
+        at += c
+    assert at == len(tokens)
+    if finish:
+        eng.trace_finish(rid)
+    return np.concatenate(rows, 0)
+
+
+def deviation(got, want):
+    """Largest row deviation as a fraction of the logits' root mean square."""
+    want = np.asarray(want, dtype=np.float64)
+    return float(np.sqrt(((got - want) ** 2).mean(-1)).max() / np.sqrt((want ** 2).mean()))
+
+
+def close(got, want, dtype):
+    """Whether the engine's rows are the plain implementation's.  In float32 every row, to a few units of rounding.  In
+    bfloat16 the router sees a rounded input, and where two experts' logits all but tie it may choose the other one: nine
+    rows in ten must lie within what rounding costs, and none may be far off."""
+    want = np.asarray(want, dtype=np.float64)
+    rows = np.sqrt(((got - want) ** 2).mean(-1)) / np.sqrt((want ** 2).mean())
+    if dtype == "float32":
+        return bool(rows.max() < TOLERANCE[dtype])
+    return bool(np.quantile(rows, 0.9) < TOLERANCE[dtype] and rows.max() < 0.5)
+
+
+def plain_logits(cfg, w, tokens):
+    return plain.forward(cfg, w, tokens).numpy()
+
+
+# ------------------------------------------------------------------------------------------ each mechanism alone
+SMALL_MIXER = gla(1, 4, 4)            # a small mixer under the feed-forward that is tested
+ALONE = {
+    "attention": config([layer("attention", attention(4, 2, 16, 16, size=12, rot_dims=8), None)], width=32, vocab=50),
+    "attention_whole_head_rotation": config([layer("attention", attention(2, 1, 32, 32, size=9, rot_dims=32, base=77.0), None)], width=32, vocab=50),
+    "attention_wide_values_wide_window": config([layer("attention", attention(2, 2, 8, 48, size=500, rot_dims=4), None)], width=32, vocab=50),
+    "attention_keys_wider_than_values": config([layer("attention", attention(3, 3, 40, 24, size=20, rot_dims=20), None)], width=32, vocab=50),
+    "attention_window_of_one": config([layer("attention", attention(2, 1, 16, 16, size=1, rot_dims=16, scale=1.0), None)], width=32, vocab=50),
+    "attention_on_the_keys_of_another": config([layer("attention", attention(2, 1, 16, 24, size=6, rot_dims=8), None),
+                                                layer("gla", SMALL_MIXER, None),
+                                                layer("attention", attention(4, 1, 16, 24, size=21, rot_dims=8, scale=0.5, kv_from=0), None),
+                                                layer("attention", attention(2, 1, 16, 24, size=3, rot_dims=8, kv_from=0), None)], width=32, vocab=50),
+    "linear_attention": config([layer("gla", gla(4, 8, 16, tau=8.0), None)], width=32, vocab=50),
+    "linear_attention_one_head_root_of_one": config([layer("gla", gla(1, 24, 24, tau=1.0), None)], width=32, vocab=50),
+    "linear_attention_wide_keys": config([layer("gla", gla(2, 100, 40, tau=2.5), None)], width=32, vocab=50),
+    "linear_attention_alone_in_the_model": config([layer("gla", gla(2, 16, 8), moe(3, 1, 8)), layer("gla", gla(3, 8, 8), None)], width=32, vocab=50),
+    "experts": config([layer("gla", SMALL_MIXER, moe(7, 2, 20, limit=1.0))], width=32, vocab=50, embed_scale=1.0),
+    "experts_all_chosen_and_shared": config([layer("gla", SMALL_MIXER, moe(4, 4, 56, limit=0.6, shared=(24, 0.4)))], width=32, vocab=50),
+    "experts_many_of_one": config([layer("gla", SMALL_MIXER, moe(70, 1, 8, shared=(72, 5.0)))], width=32, vocab=50),
+    "no_cap_on_the_logits": config([layer("attention", attention(2, 2, 16, 16, size=5, rot_dims=2), moe(2, 1, 8))], width=32, vocab=50, softcap=None),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(ALONE))
+def test_each_mechanism_alone(tmp_path, name, dtype):
+    cfg = copy.deepcopy(ALONE[name])
+    if cfg["logit_softcap"] is None:
+        del cfg["logit_softcap"]
+    w = random_weights(cfg, 3, rank=5)
+    folder = write_model(tmp_path / name, cfg, w)
+    tokens = tokens_for(cfg, 45, 1)
+    want = plain_logits(cfg, w, tokens)
+    eng = engine(folder, dtype)
+    assert close(run_cut(eng, 0, tokens, [45]), want, dtype)
+    assert close(run_cut(eng, 1, tokens, [9, 2, 17] + [1] * 17), want, dtype)
+
+
+def test_many_rows_an_expert_take_the_tile_product(tmp_path):
+    """A prompt long enough that the experts' rows go through the grouped tile product, its tokens one by one through the
+    other route: the same logits."""
+    cfg = config([layer("gla", SMALL_MIXER, moe(2, 1, 64, limit=1.0, shared=(64, 1.0)))], width=64, vocab=50)
+    w = random_weights(cfg, 4)
+    folder = write_model(tmp_path / "tiles", cfg, w)
+    tokens = tokens_for(cfg, 160, 2)
+    for dtype in ("float32", "bfloat16"):
+        eng = engine(folder, dtype)
+        whole = run_cut(eng, 0, tokens, [160])
+        assert close(whole, plain_logits(cfg, w, tokens), dtype)
+        assert deviation(run_cut(eng, 1, tokens, [100] + [1] * 60), whole) < SAME[dtype]
+
+
+def test_the_residual_stream_is_32_bit(tmp_path):
+    """Many layers with small updates on a large embedding: a stream rounded to 16 bits between layers would lose them."""
+    cfg = config([layer("gla", SMALL_MIXER, None) for _ in range(12)], width=32, vocab=40, embed_scale=40.0)
+    w = random_weights(cfg, 5)
+    for n in w:
+        if n.endswith("norm1b"):
+            w[n] = torch.full_like(w[n], -0.95)         # the weight that multiplies is 1 + w
+    w["embed"] = (w["embed"].float() * 40.0).to(torch.bfloat16)
+    folder = write_model(tmp_path / "deep", cfg, w)
+    tokens = tokens_for(cfg, 20, 2)
+    got = run_cut(engine(folder, "bfloat16"), 0, tokens, [20])
+    assert deviation(got, plain_logits(cfg, w, tokens)) < 1.5e-2
+
+
+# ----------------------------------------------------------------------------- cuttings, batches, pages and slots
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_whole_prompt_portions_and_decoding_agree(models, name, dtype):
+    folder, cfg, w = models[name]
+    n = 150
+    tokens = tokens_for(cfg, n, 7)
+    want = plain_logits(cfg, w, tokens)
+    eng = engine(folder, dtype, page_size=16 if name == "MIXED" else 64)
+    whole = run_cut(eng, 0, tokens, [n])
+    assert close(whole, want, dtype)
+    # The first tokens of a sequence on their own rows.
+    assert deviation(whole[:4], want[:4]) < TOLERANCE[dtype] * (1 if dtype == "float32" else 3)
+    cuttings = {
+        "token by token": [1] * n,
+        "portions down to two tokens": [2, 3, 16, 2, 1, 31, 2, 33, 5, 1, 1, 2, 17, 32, 2],
+        "a prompt and then decoding": [n - 60] + [1] * 60,
+        "portions that end on page borders": [16, 48, 64, 22],
+    }
+    for what, cuts in cuttings.items():
+        got = run_cut(eng, 1, tokens, cuts)
+        assert deviation(got, whole) < SAME[dtype], what
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_unequal_requests_in_one_batch(models, dtype):
+    """Portions of some requests beside single tokens of others, a request left out of a step, against each alone."""
+    folder, cfg, w = models["MIXED"]
+    lengths = [70, 23, 41, 5]
+    seqs = [tokens_for(cfg, n, 30 + i) for i, n in enumerate(lengths)]
+    eng = engine(folder, dtype)
+    alone = [run_cut(eng, 10 + i, s, [len(s)]) for i, s in enumerate(seqs)]
+    at = [0] * 4
+    got = [[] for _ in seqs]
+    step = 0
+    while any(a < n for a, n in zip(at, lengths)):
+        entries, who = [], []
+        for i, s in enumerate(seqs):
+            if at[i] >= lengths[i] or (step + i) % 5 == 4:        # finished, or left out of this step
+                continue
+            c = min([7, 1, 2, 1][(step + i) % 4], lengths[i] - at[i])
+            entries.append((i, s[at[i]:at[i] + c], list(range(c))))
+            who.append((i, c))
+            at[i] += c
+        step += 1
+        if not entries:
+            continue
+        rows = eng.trace_step(entries)
+        r = 0
+        for i, c in who:
+            got[i].append(rows[r:r + c])
+            r += c
+    for i in range(4):
+        assert deviation(np.concatenate(got[i], 0), alone[i]) < SAME[dtype], i
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_and_slots_are_used_again(models, dtype):
+    """A pool of one request's pages and one state slot: every request starts in what the one before left."""
+    folder, cfg, w = models["MIXED"]
+    eng = engine(folder, dtype, num_pages=5, page_size=16, max_num_seqs=1)
+    for i, n in enumerate([60, 17, 64, 33]):
+        tokens = tokens_for(cfg, n, 50 + i)
+        got = run_cut(eng, i, tokens, [n // 2, n - n // 2 - 3, 1, 1, 1])
+        assert close(got, plain_logits(cfg, w, tokens), dtype), i
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_past_many_windows(models, dtype):
+    """Pages behind every window are given back on the way: a pool far smaller than the sequence suffices."""
+    folder, cfg, w = models["MIXED"]
+    n = 300
+    tokens = tokens_for(cfg, n, 9)
+    eng = engine(folder, dtype, num_pages=8)
+    got = run_cut(eng, 0, tokens, [40] + [1] * (n - 40))
+    assert close(got, plain_logits(cfg, w, tokens), dtype)
+
+
+# ------------------------------------------------------------------------------- a key that stands out, at every edge
+def marked_attention_model(size, reader_size=None, head=16):
+    """One layer whose attention has one head whose query and key are constant directions, so that every query scores
+    high on a key wherever that key's token is the mark (token 1) and about zero elsewhere, and whose value carries the
+    mark into the logits: the logits move if and only if the marked key is visible.  With reader_size, the first layer's
+    output is switched off and a second layer with that window reads the first layer's keys."""
+    layers = [layer("attention", attention(1, 1, head, head, size=size, rot_dims=2, base=1e6, scale=1.0), None)]
+    if reader_size:
+        layers.append(layer("attention", attention(1, 1, head, head, size=reader_size, rot_dims=2, base=1e6, scale=1.0, kv_from=0), None))
+    cfg = config(layers, width=32, vocab=12, embed_scale=1.0)
+    w = random_weights(cfg, 77)
+    W = cfg["width"]
+    embed = torch.zeros(12, W)
+    embed[:, 0] = 1.0                      # every token: a constant channel that makes the query
+    embed[1, 1] = 6.0                      # the mark: a channel that makes the key and the value
+    embed[2:, 2:] = torch.randn(10, W - 2, generator=torch.Generator().manual_seed(3)) * 0.2
+    w["embed"] = embed.to(torch.bfloat16)
+    q = torch.zeros(head, W)
+    k = torch.zeros(head, W)
+    v = torch.zeros(head, W)
+    q[head - 1, 0] = 1.0                   # the last dimension of the head is not rotated; the head norm makes it sqrt(head)
+    k[head - 1, 1] = 1.0                   # a key's last dimension: sqrt(head) for the mark, 0 for any other token
+    v[:, 1] = 1.0
+    for i in range(len(layers)):
+        p = f"l{i}."
+        w[p + "norm1"] = torch.zeros(W).to(torch.bfloat16)
+        w[p + "mix.q"] = q.to(torch.bfloat16)
+        w[p + "mix.q.norm"] = torch.ones(head).to(torch.bfloat16)
+        w[p + "mix.g"] = torch.zeros(head, W).to(torch.bfloat16)        # every gate is one half
+    w["l0.mix.k"], w["l0.mix.v"] = k.to(torch.bfloat16), v.to(torch.bfloat16)
+    w["l0.mix.k.norm"] = torch.ones(head).to(torch.bfloat16)
+    if reader_size:
+        w["l0.norm1b"] = torch.full((W,), -1.0).to(torch.bfloat16)       # 1 + w = 0: the first layer adds nothing
+    return cfg, w
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("reader", [None, 40, 9])
+def test_a_marked_key_is_seen_exactly_inside_the_window(tmp_path, dtype, reader):
+    """reader: a second layer with a window of its own (wider or narrower than the first's) on the first layer's keys."""
+    size, page = 24, 16
+    seen = reader or size
+    cfg, w = marked_attention_model(size, reader)
+    folder = write_model(tmp_path / "marked", cfg, w)
+    eng = engine(folder, dtype, num_pages=16, page_size=page)
+    n = 100
+    rid = 0
+    # (marked position, asking position): both edges of the window, at page borders, far away, the first tokens.
+    cases = [(0, 0), (0, seen - 1), (0, seen), (1, seen), (1, seen + 1), (40, 40), (40, 39 + seen), (40, 40 + seen), (31, 32), (32, 47), (47, 48),
+             (5, 95), (95 - seen, 95), (96 - seen, 95), (95, 95), (96, 99), (95, 96), (15, 16), (16, 16 + seen - 1), (16, 16 + seen)]
+    for mark, ask in cases:
+        if ask >= n:
+            continue
+        tokens = [2 + (i * 7) % 10 for i in range(n)]
+        base = list(tokens)
+        tokens[mark] = 1
+        visible = 0 <= ask - mark < seen
+        p_marked = plain_logits(cfg, w, tokens)[ask]
+        p_base = plain_logits(cfg, w, base)[ask]
+        moved = np.abs(p_marked - p_base).max()
+        if mark != ask:
+            assert (moved > 0.05) == visible, (mark, ask, moved)        # the plain implementation itself, first
+        for cuts in ([n], [ask] + [1] * (n - ask) if ask else [n], [mark + 1, n - mark - 1] if mark + 1 < n else [n], [3, 2] + [5] * 19):
+            got = run_cut(eng, rid, tokens, cuts)[ask]
+            rid += 1
+            assert np.sqrt(((got - p_marked) ** 2).mean()) < TOLERANCE[dtype] * np.sqrt((p_marked ** 2).mean()) + 1e-3, (mark, ask, cuts[:3])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_constant_in_the_denominator(tmp_path, dtype):
+    """Scores far below zero: without the 1 in the denominator the weights would still sum to 1 and the output would be a
+    mean of values; with it the output all but vanishes."""
+    cfg, w = marked_attention_model(50)
+    w["l0.mix.q"] = (-w["l0.mix.q"].float()).to(torch.bfloat16)
+    folder = write_model(tmp_path / "sink", cfg, w)
+    tokens = [1] * 30
+    want = plain_logits(cfg, w, tokens)
+    got = run_cut(engine(folder, dtype), 0, tokens, [30])
+    assert close(got, want, dtype)
+    # The plain implementation itself: the same scores through an ordinary softmax give another answer.
+    x = w["embed"].double()[torch.tensor(tokens)]
+    h = plain.norm_around_zero(x, w["l0.norm1"], cfg["norm"]["eps"])
+    out, _ = plain.attention(cfg["layers"][0]["mixer"], w, "l0.mix.", h, cfg["norm"]["eps"])
+    ordinary = (0.5 * (h[:1] @ w["l0.mix.v"].double().T)) @ w["l0.mix.o"].double().T      # all tokens are equal: the mean of the values is any of them
+    assert out.abs().max() < 0.01 * ordinary.abs().max()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_recurrence_cut_between_any_two_tokens(tmp_path, dtype):
+    cfg = config([layer("gla", gla(2, 16, 16, tau=3.0), None), layer("gla", gla(4, 8, 24), moe(4, 2, 16))], width=32, vocab=50)
+    w = random_weights(cfg, 8)
+    folder = write_model(tmp_path / "cuts", cfg, w)
+    n = 40
+    tokens = tokens_for(cfg, n, 4)
+    eng = engine(folder, dtype)
+    whole = run_cut(eng, 0, tokens, [n])
+    assert close(whole, plain_logits(cfg, w, tokens), dtype)
+    for cut in range(1, n):
+        assert deviation(run_cut(eng, cut, tokens, [cut, n - cut]), whole) < SAME[dtype], cut
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_slow_decay_remembers_the_first_token(tmp_path, dtype):
+    """A decay near one keeps the first token's key and value for hundreds of tokens: a state that is lost or reset on the
+    way shows in the last logits."""
+    cfg = config([layer("gla", gla(1, 8, 8, tau=64.0), None)], width=32, vocab=20)
+    w = random_weights(cfg, 12)
+    w["l0.mix.a2.b"] = torch.full_like(w["l0.mix.a2.b"], 6.0)
+    folder = write_model(tmp_path / "slow", cfg, w)
+    n = 260
+    a = tokens_for(cfg, n, 5)
+    b = list(a)
+    b[0] = (a[0] + 1) % cfg["vocab"]
+    want_a, want_b = plain_logits(cfg, w, a), plain_logits(cfg, w, b)
+    assert np.abs(want_a[-1] - want_b[-1]).max() > 0.01          # the plain implementation: the first token still matters
+    eng = engine(folder, dtype, num_pages=20)
+    for tokens, want in ((a, want_a), (b, want_b)):
+        assert close(run_cut(eng, 0, tokens, [100, 7] + [1] * (n - 107)), want, dtype)
+
+
+# ------------------------------------------------------------------------------------------------- generation
+@pytest.mark.parametrize("graphs", [False, True])
+def test_greedy_generation_through_the_scheduler(models, graphs):
+    """create_engine -> the scheduler, the step function, the sampler: the tokens are the plain implementation's."""
+    from vosti_amd.engine import create_engine
+    from vosti_amd.sampling.params import SamplingParams
+    folder, cfg, w = models["MIXED"]
+    prompts = [tokens_for(cfg, n, 60 + i) for i, n in enumerate([19, 3, 40])]
+    eng = create_engine(folder, dtype="float32", num_pages=24, page_size=16, max_num_seqs=4, graphs=graphs)
+    out = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    for prompt, got in zip(prompts, out):
+        assert list(got) == plain.generate_greedy(cfg, w, prompt, 12)
