@@ -6,6 +6,7 @@
     python bench.py --workload mixed14b     # Qwen3-14B shape: 32 prompts of 128 to 4,096 tokens, prefill in portions beside decoding
     python bench.py --workload prefix32b    # Qwen3-32B shape: 64 requests at context 8,192 that share a 1,024-token prefix
     python bench.py --workload aligned      # the reference's aligned phases: batch 4, cached contexts 0 to 16K, 256 new tokens / 127 decode steps
+    python bench.py --workload pabavik      # the Pabavik design (gated linear attention, windowed attention with an output gate, gated experts beside a shared one) at three layer sizes beside Tezinex at equal size
     python bench.py --workload povatar      # the Povatar design (attention beside a state-space recurrence, routed experts) at three layer sizes beside Tezinex at equal size
     python bench.py --workload tezinex      # the Tezinex design at three layer sizes beside the Qwen3 decoder at equal size: prefill and decode
 
@@ -87,9 +88,9 @@ def main() -> int:
     ap.add_argument("--no-other-shapes", action="store_true", help="skip the 14B and 32B workloads that the default record holds as points")
     ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
                     help="context length of the decode measurement (the prefill figure is always of 2,048 tokens)")
-    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b", "aligned", "tezinex", "povatar"])
-    ap.add_argument("--sizes", default=",".join(["1k", "2k", "4k"]), help="which layer sizes --workload tezinex / povatar measure (1k, 2k, 4k)")
-    ap.add_argument("--only-design", default="", choices=["", "tezinex", "qwen3", "povatar"], help="--workload tezinex / povatar: measure one of the two designs only")
+    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b", "aligned", "tezinex", "povatar", "pabavik"])
+    ap.add_argument("--sizes", default=",".join(["1k", "2k", "4k"]), help="which layer sizes --workload tezinex / povatar / pabavik measure (1k, 2k, 4k)")
+    ap.add_argument("--only-design", default="", choices=["", "tezinex", "qwen3", "povatar", "pabavik"], help="--workload tezinex / povatar / pabavik: measure one of the two designs only")
     ap.add_argument("--engine", default="native", choices=["native", "python"],
                     help="which engine every figure is measured through: the native one (vosti_amd.engine.NativeEngine) or the "
                          "Python step function over the same kernels, cache manager and scheduler")
@@ -112,7 +113,7 @@ def main() -> int:
     if args.workload == "aligned":
         print(json.dumps(aligned_workload(args)), flush=True)
         return 0
-    if args.workload in ("tezinex", "povatar"):
+    if args.workload in ("tezinex", "povatar", "pabavik"):
         print(json.dumps(tezinex_workload(args)), flush=True)
         return 0
     if args.workload != "decode8b":
@@ -545,10 +546,32 @@ def povatar_config(width, heads, kv_heads, ff, layers, vocab):
             "layers": [{"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp} for _ in range(layers)]}
 
 
+def pabavik_config(width, heads, kv_heads, ff, layers, vocab):
+    """Linear attention, attention, attention on the keys of the one before, linear attention, ... (Tezinex's order of
+    layers, with the same heads of 128, the same window and a state of the same size), every layer with 32 experts a
+    quarter as wide as the dense feed-forward of the same size, of which a token uses 3, beside a shared one of that
+    width: a token's matrix work is that of a Tezinex or Qwen3 layer of these sizes."""
+    def attention(kv_from=None):
+        m = {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": kv_heads, "mask": {"size": 1024}, "scale": 128 ** -0.5,
+             "rot": {"base": 10000.0, "dims": 64}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return {"type": "attention", "mixer": m, "mlp": mlp}
+    mlp = {"kind": "moe", "expert": {"ff": ff // 4, "limit": 7.0}, "router": {"experts": 32, "top": 3}, "shared": {"ff": ff // 4, "limit": 7.0}}
+    linear = {"type": "gla", "mixer": {"dim": 128, "vdim": 128, "heads": heads, "tau": 16.0}, "mlp": mlp}
+    out = []
+    for i in range(layers):
+        kind = i % 4
+        out.append(linear if kind in (0, 3) else attention(i - 1 if kind == 2 else None))
+    return {"architecture": "Pabavik", "embedding": {"scale": 1.0}, "layers": out, "logit_softcap": 20.0, "norm": {"eps": 1e-5}, "vocab": vocab,
+            "width": width}
+
+
 def tezinex_workload(args) -> dict:
     """Prefill of one prompt and decoding at a fixed batch for the Tezinex design at three layer sizes, each beside the
     Qwen3 decoder with the same width, heads, feed-forward, layers and vocabulary (random weights, the native engine).
-    --workload povatar: the Povatar design beside Tezinex, its nearest neighbour here, in the same way."""
+    --workload povatar: the Povatar design beside Tezinex, its nearest neighbour here, in the same way; --workload pabavik:
+    the Pabavik design beside Tezinex."""
     import tempfile
     from vosti_amd.engine import NativeEngine
     from vosti_amd.sampling import SamplingParams
@@ -560,7 +583,8 @@ def tezinex_workload(args) -> dict:
     record = {"metric": "decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
               "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
               "data": "synthetic: seeded random token prompts, seeded random weights", "sizes": {},
-              "config": {"model": "Povatar (attention beside a state-space recurrence, 32 experts of which 4) beside Tezinex at equal size"
+              "config": {"model": "Pabavik (linear attention, attention, shared-key attention, linear attention, ...; 32 experts of which 3 and a shared one) beside Tezinex at equal size"
+                         if args.workload == "pabavik" else "Povatar (attention beside a state-space recurrence, 32 experts of which 4) beside Tezinex at equal size"
                          if args.workload == "povatar" else "Tezinex (delta, attention, shared-key attention, delta, ...) beside Qwen3 at equal size",
                          "layers": layers,
                          "global_batch": batch, "seq_len": prompt_tokens, "vocab_size": vocab, "parallelism": "single GPU",
@@ -605,11 +629,13 @@ def tezinex_workload(args) -> dict:
                     "decode_ms_per_step": round(step_s * 1e3, 4), "decode_tokens_per_s": round(batch / step_s, 1)}
 
     # The design that is measured and the neighbour it stands beside.
-    first, second = ("povatar", "tezinex") if args.workload == "povatar" else ("tezinex", "qwen3")
+    first, second = (args.workload, "tezinex") if args.workload in ("povatar", "pabavik") else ("tezinex", "qwen3")
 
     def config_of(design, width, heads, kv_heads, ff):
         if design == "povatar":
             return povatar_config(width, heads, kv_heads, ff, layers, vocab)
+        if design == "pabavik":
+            return pabavik_config(width, heads, kv_heads, ff, layers, vocab)
         if design == "tezinex":
             return tezinex_config(width, heads, kv_heads, ff, layers, vocab)
         return dict(QWEN3_8B, architectures=["Qwen3ForCausalLM"], vocab_size=vocab, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
