@@ -154,7 +154,9 @@ ModelSpec pabavik_model_spec(const Json& raw) {
     if (const Json* mlp = present(l, "mlp")) {
       const std::string mw = where + " mlp";
       const Json* kind = mlp->get("kind");
-      if (!kind || kind->kind != Json::String || kind->text != "moe") throw ConfigError("config.json: " + where + ": the feed-forward's 'kind' must be 'moe'");
+      // The design has one kind of feed-forward; a configuration that names none means that one.
+      if (kind && kind->kind != Json::Null && (kind->kind != Json::String || kind->text != "moe"))
+        throw ConfigError("config.json: " + where + ": the feed-forward's 'kind' must be 'moe'");
       const Json& router = member(*mlp, "router", mw);
       const int64_t experts = positive(router, "experts", mw + ".router"), top = positive(router, "top", mw + ".router");
       if (top > experts) throw ConfigError("config.json: " + where + ": 'top' must not exceed 'experts'");
