@@ -348,3 +348,59 @@ def test_greedy_generation_through_the_scheduler(models, graphs):
     out = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
     for prompt, got in zip(prompts, out):
         assert list(got) == plain.generate_greedy(cfg, w, prompt, 12)
+
+
+# --------------------------------------------------------------------------------------------- the replay program
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_replay_program_with_four_slots_and_a_pool_for_the_live_requests(models, tmp_path, dtype):
+    """bin/trace_run as a user starts it: six requests of which at most four are live, portions of prompts beside single
+    tokens, requests left out of steps, a pool sized for the live requests alone (so that pages and state slots are used
+    again), a name that comes back after its request ended.  Every row against the plain implementation."""
+    import json
+    import random
+    import subprocess
+    import sys
+    from pathlib import Path
+    folder, cfg, w = models["MIXED"]
+    lengths = {"a": 70, "b": 33, "c": 150, "d": 9, "e": 64, "f": 101, "a again": 41}
+    tokens = {name: tokens_for(cfg, n, 80 + i) for i, (name, n) in enumerate(lengths.items())}
+    rng = random.Random(5)
+    waiting, live, fed, steps, most = list(lengths), [], {}, [], 0
+    while waiting or live:
+        while waiting and len(live) < 4 and not (waiting[0] == "a again" and "a" in live):
+            live.append(waiting.pop(0))
+            fed[live[-1]] = 0
+        most = max(most, sum(-(-lengths[n] // 64) * 64 for n in live))
+        entries, end = [], []
+        for name in list(live):
+            if rng.random() < 0.2 and len(live) > 1:
+                continue                                            # left out of this step
+            left = lengths[name] - fed[name]
+            size = min(left, 1 if left <= 6 else rng.choice([1, 2, 3, 7, 16, 40]))
+            entries.append({"id": name.split()[0], "name": name, "tokens": tokens[name][fed[name]:fed[name] + size], "want": list(range(size))})
+            fed[name] += size
+            if fed[name] == lengths[name]:
+                end.append(name.split()[0])
+                live.remove(name)
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+    cmd = [sys.executable, str(Path(__file__).resolve().parent.parent / "bin" / "trace_run"), "--model", str(folder), "--dtype", dtype,
+           "--out", str(tmp_path), "--max-tokens", str(most)]
+    proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    for rec in steps:
+        proc.stdin.write(json.dumps(rec) + "\n")
+        proc.stdin.flush()
+        assert proc.stdout.readline().strip() == f"done {rec['step']}"
+    proc.stdin.close()
+    assert proc.wait(timeout=60) == 0
+    rows = {name: [] for name in lengths}
+    for rec in steps:
+        if not any(e["want"] for e in rec["entries"]):
+            continue
+        got = np.fromfile(tmp_path / f"{rec['step']}.f32", dtype="<f4").reshape(-1, cfg["vocab"])
+        at = 0
+        for e in rec["entries"]:
+            rows[e["name"]].append(got[at:at + len(e["want"])])
+            at += len(e["want"])
+        assert at == got.shape[0]
+    for name in lengths:
+        assert close(np.concatenate(rows[name], 0), plain_logits(cfg, w, tokens[name]), dtype), name
