@@ -50,8 +50,8 @@ MIXED = config([
     layer("attention", attention(8, 1, 16, 16, size=64, rot_dims=4, base=77.0, kv_from=3), moe(4, 1, 8, shared=(8, 1.0))),
 ], width=64, vocab=97)
 # One layer of each kind with the head size of the kernels' widest tiles, and a state as wide as a wave.
-WIDE = config([layer("attention", attention(4, 2, 128, 128, size=150, rot_dims=32, base=250000.0), moe(8, 2, 72, shared=(136, 1.0))),
-               layer("gla", gla(2, 64, 64), moe(8, 4, 64, limit=1.5)),
+WIDE = config([layer("attention", attention(4, 2, 128, 128, size=150, rot_dims=32, base=250000.0), moe(8, 2, 72, shared=(120, 0.9))),
+               layer("gla", gla(2, 64, 64), moe(12, 5, 64, limit=1.25)),
                layer("attention", attention(4, 2, 128, 128, size=70, rot_dims=32, base=250000.0, kv_from=0), None)], width=96, vocab=130, embed_scale=9.0)
 CONFIGS = {"MIXED": MIXED, "WIDE": WIDE}
 RANK = 6      # of the decay's two projections; no key of the configuration holds it
