@@ -153,13 +153,15 @@ struct RuleShape {
 
 //
 // DELTA false is the same walk without the correction: S <- diag(g) S + k v^T; o = S^T q (gated linear attention); beta is
-// not read, q is multiplied by q_scale as it is brought in, and the inputs may be elements (IN).
+// not read, q is multiplied by q_scale as it is brought in, and the inputs may be elements (IN).  head_decay: one decay a
+// head [H] that takes the place of the decays per token and channel; in_act 1: q, k and v pass silu as they are brought in.
 template <int R, int DR, bool DELTA, typename IN>
 __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restrict__ out, const IN* __restrict__ qkv, int64_t ld, int q_col,
                                                                   int k_col, int v_col, const float* __restrict__ decay,
                                                                   const elem_t* __restrict__ b, int64_t ldb, float* state, int64_t state_stride,
                                                                   const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
-                                                                  const int32_t* __restrict__ slots, int H, int G, int d, int dv, float q_scale) {
+                                                                  const int32_t* __restrict__ slots, int H, int G, int d, int dv, float q_scale,
+                                                                  const float* __restrict__ head_decay, int in_act) {
   using Sh = RuleShape<R, DR>;
   constexpr int DMAX = Sh::DMAX, TC = Sh::TC, CB = Sh::CB;
   __shared__ __attribute__((aligned(16))) float smem[2 * Sh::BUF];
@@ -205,8 +207,13 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
       const bool ok = e < TC * DMAX && t0 + tok < n && c < d;
       const int64_t t = first + t0 + (ok ? tok : 0);
       const int cc = ok ? c : 0;
-      const float kv = to_f32(qkv[t * ld + k_col + (int64_t)g * d + cc]), qv = to_f32(qkv[t * ld + q_col + (int64_t)g * d + cc]);
-      const float gv = decay[(t * H + h) * d + cc];
+      float kv = to_f32(qkv[t * ld + k_col + (int64_t)g * d + cc]), qv = to_f32(qkv[t * ld + q_col + (int64_t)g * d + cc]);
+      if (in_act) {
+        kv = silu_f(kv);
+        qv = silu_f(qv);
+      }
+      // One decay a head for all tokens and channels, or one per token and channel.
+      const float gv = head_decay != nullptr ? head_decay[h] : decay[(t * H + h) * d + cc];
       pk[it] = ok ? kv : 0.f;
       pq[it] = ok ? (DELTA ? qv : qv * q_scale) : 0.f;
       pg[it] = ok ? gv : 1.f;
@@ -218,7 +225,7 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
       const bool ok = e < TC * CB && t0 + tok < n && blockIdx.z * CB + c < dv;
       const int64_t t = first + t0 + (ok ? tok : 0);
       const float vv = to_f32(qkv[t * ld + v_col + (int64_t)h * dv + (ok ? blockIdx.z * CB + c : 0)]);
-      pv[it] = ok ? vv : 0.f;
+      pv[it] = ok ? (in_act ? silu_f(vv) : vv) : 0.f;
     }
     if (DELTA && tid < TC) {
       const bool ok = t0 + tid < n;
@@ -409,8 +416,9 @@ extern "C++" {
 template <bool DELTA, typename IN>
 static int rule_launch(float* out, const IN* qkv, int64_t ld, int q_col, int k_col, int v_col, const float* decay, const elem_t* b, int64_t ldb,
                        float* state, int64_t state_stride, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int G,
-                       int d, int dv, float q_scale, hipStream_t st) {
+                       int d, int dv, float q_scale, hipStream_t st, const float* head_decay = nullptr, int in_act = 0) {
   VK_REQUIRE(S >= 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0, "delta rule: bad sizes H=%d G=%d d=%d dv=%d", H, G, d, dv);
+  VK_REQUIRE((decay != nullptr) != (head_decay != nullptr), "delta rule: decays per token and channel, or one a head");
   VK_REQUIRE(d <= 1024, "delta rule: key size %d exceeds 1024", d);
   VK_REQUIRE(state_stride >= (int64_t)H * d * dv, "delta rule: the state is too small");
   if (S == 0) return 0;
@@ -419,7 +427,7 @@ static int rule_launch(float* out, const IN* qkv, int64_t ld, int q_col, int k_c
   const dim3 grid(S, H, (dv + cols - 1) / cols);
   VK_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "delta rule: too many heads or columns");
 #define RULE(RR, DD) \
-  delta_rule_kernel<RR, DD, DELTA, IN><<<grid, RULE_THREADS, 0, st>>>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, H, G, d, dv, q_scale)
+  delta_rule_kernel<RR, DD, DELTA, IN><<<grid, RULE_THREADS, 0, st>>>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, H, G, d, dv, q_scale, head_decay, in_act)
   if (DR == 4) {
     switch (R) {
       case 1: RULE(1, 4); break;
@@ -463,6 +471,16 @@ int vk_gla_rule(float* out, const elem_t* x, int64_t ld, int q_col, int k_col, i
                 const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int d, int dv, float q_scale, hipStream_t st) {
   return rule_launch<false, elem_t>(out, x, ld, q_col, k_col, v_col, decay, nullptr, 0, state, state_stride, cu_q, positions, slots, S, H, H, d, dv,
                                     q_scale, st);
+}
+
+// Linear attention with one fixed decay a head: S <- decay[h] S + k v^T, o = S^T q with q = silu(.), k = silu(.), v = silu(.)
+// of the elements at the three columns of x (in_act 1; 0: the elements as they are), q times q_scale.  decay [H] floats.
+int vk_linear_rule(float* out, const elem_t* x, int64_t ld, int q_col, int k_col, int v_col, const float* head_decay, int in_act, float* state,
+                   int64_t state_stride, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int d, int dv, float q_scale,
+                   hipStream_t st) {
+  VK_REQUIRE(head_decay != nullptr && (in_act == 0 || in_act == 1), "linear attention: the heads' decays are missing");
+  return rule_launch<false, elem_t>(out, x, ld, q_col, k_col, v_col, nullptr, nullptr, 0, state, state_stride, cu_q, positions, slots, S, H, H, d, dv,
+                                    q_scale, st, head_decay, in_act);
 }
 
 int vk_delta_out(elem_t* y, int64_t ldy, const float* o, const elem_t* gate, int64_t ldg, const void* w, int w_is_f32, int T, int H, int dv,

@@ -140,9 +140,18 @@ struct Kernels::Fn {
   int (*moe_glu)(P, CP, int64_t, int, float, float, float, hipStream_t);
   int (*moe_combine_add)(P, CP, CP, CP, CP, int, int, int, hipStream_t);
   int (*stream_norm_add_f32)(P, CP, CP, CP, int, int, int, float, float, float, hipStream_t);
+  int (*cast_from_f32)(P, CP, int64_t, hipStream_t);
+  int (*moe_route_scored)(P, P, P, CP, CP, CP, int, int, int, int, int, float, int, hipStream_t);
+  int (*moe_glu_weighed)(P, CP, int64_t, int, float, float, float, CP, CP, hipStream_t);
+  int (*norm_columns)(P, int64_t, CP, int64_t, int, int, CP, int, float, int, hipStream_t);
+  int (*gemm_heads)(P, int64_t, int64_t, CP, int64_t, int64_t, CP, int, int, int, int, hipStream_t);
+  int (*latent_post)(CP, int64_t, CP, int64_t, int64_t, int, P, P, P, CP, int, float, CP, int, CP, CP, int, int, int, int, int, int, hipStream_t);
+  int (*qkv_post_norm_angles_paired)(CP, int64_t, P, P, P, CP, CP, int, int, float, CP, float, int, int, CP, CP, int, int, int, int, int, hipStream_t);
+  int (*linear_rule)(P, CP, int64_t, int, int, int, CP, int, P, int64_t, CP, CP, CP, int, int, int, int, float, hipStream_t);
+  int (*side_gate)(P, int64_t, CP, int64_t, CP, int64_t, CP, int, int, int, hipStream_t);
 };
 
-static constexpr int KERNEL_ABI = 17;
+static constexpr int KERNEL_ABI = 18;
 
 Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(name), fn_(new Fn) {
   if (name == "bf16") dtype_ = DType::BF16;
@@ -180,6 +189,9 @@ Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(na
   VK(qkv_post_norm_angles, "vk_qkv_post_norm_angles"); VK(gate_mul, "vk_gate_mul"); VK(gla_decay, "vk_gla_decay"); VK(gla_rule, "vk_gla_rule");
   VK(gated_head_norm, "vk_gated_head_norm"); VK(moe_route_bias, "vk_moe_route_bias"); VK(moe_up_plain, "vk_moe_up_plain"); VK(moe_glu, "vk_moe_glu");
   VK(moe_combine_add, "vk_moe_combine_add"); VK(stream_norm_add_f32, "vk_stream_norm_add_f32");
+  VK(cast_from_f32, "vk_cast_from_f32"); VK(moe_route_scored, "vk_moe_route_scored"); VK(moe_glu_weighed, "vk_moe_glu_weighed");
+  VK(norm_columns, "vk_norm_columns"); VK(gemm_heads, "vk_gemm_heads"); VK(latent_post, "vk_latent_post");
+  VK(qkv_post_norm_angles_paired, "vk_qkv_post_norm_angles_paired"); VK(linear_rule, "vk_linear_rule"); VK(side_gate, "vk_side_gate");
 #undef VK
   segment_keys_ = fn_->attn_segment_keys();
   item_rows_ = fn_->attn_item_rows();
@@ -279,6 +291,14 @@ Tensor Kernels::to_f32(const Tensor& x) {
   expect(x, "cast input", dtype_);
   Tensor out = empty(x.shape, DType::F32);
   call(fn_->cast_to_f32(out.data, x.data, x.numel(), stream));
+  return out;
+}
+
+Tensor Kernels::to_elements(const Tensor& x) {
+  expect(x, "cast input", DType::F32);
+  if (dtype_ == DType::F32) return x;
+  Tensor out = empty(x.shape);
+  call(fn_->cast_from_f32(out.data, x.data, x.numel(), stream));
   return out;
 }
 
@@ -845,6 +865,11 @@ Tensor Kernels::ssm_gate_norm(const Tensor& y, const Tensor& proj, int64_t z_col
 
 // ------------------------------------------------------------------------------ mixture of experts
 Kernels::MoePlan Kernels::moe_route(const Tensor& h, const Tensor& router, int top, float weight_eps, int tile_rows, const Tensor* bias) {
+  return moe_route_scored(h, router, top, weight_eps, tile_rows, bias, 0);
+}
+
+Kernels::MoePlan Kernels::moe_route_scored(const Tensor& h, const Tensor& router, int top, float weight_eps, int tile_rows, const Tensor* bias,
+                                           int score_kind) {
   expect(h, "router input", dtype_);
   expect(router, "router weight", dtype_);
   if (h.shape.size() != 2 || router.shape.size() != 2 || router.dim(1) != h.dim(1) || top < 1 || top > router.dim(0))
@@ -864,7 +889,11 @@ Kernels::MoePlan Kernels::moe_route(const Tensor& h, const Tensor& router, int t
   p.tile_expert = empty({tiles}, DType::I32);
   p.expert_start = empty({E + 1}, DType::I32);
   Tensor logits = empty({T, E}, DType::F32);
-  if (bias) {
+  if (score_kind != 0) {
+    const int bf = bias ? norm_weight(*bias, "router bias", E) : 0;
+    call(fn_->moe_route_scored(p.idx.data, p.wts.data, logits.data, h.data, router.data, bias ? bias->data : nullptr, bf, (int)T, (int)h.dim(1), (int)E,
+                               top, weight_eps, score_kind, stream));
+  } else if (bias) {
     const int bf = norm_weight(*bias, "router bias", E);
     call(fn_->moe_route_bias(p.idx.data, p.wts.data, logits.data, h.data, router.data, bias->data, bf, (int)T, (int)h.dim(1), (int)E, top, weight_eps,
                              stream));
@@ -921,6 +950,144 @@ Tensor Kernels::moe_glu(const Tensor& gate_up, float limit, float slope, float s
   const int64_t F = gate_up.dim(1) / 2;
   Tensor out = empty({gate_up.dim(0), F});
   call(fn_->moe_glu(out.data, gate_up.data, gate_up.dim(0), (int)F, limit, slope, shift, stream));
+  return out;
+}
+
+Tensor Kernels::moe_glu_weighed(const Tensor& gate_up, float limit, float slope, float shift, const MoePlan& plan) {
+  expect(gate_up, "gate and up outputs", dtype_);
+  if (gate_up.shape.size() != 2 || gate_up.dim(1) % 2 || gate_up.dim(0) != plan.row_pair.dim(0))
+    throw EngineError("gated activation: rows are " + gate_up.describe() + " for a plan of " + std::to_string(plan.row_pair.dim(0)) + " rows");
+  const int64_t F = gate_up.dim(1) / 2;
+  Tensor out = empty({gate_up.dim(0), F});
+  call(fn_->moe_glu_weighed(out.data, gate_up.data, gate_up.dim(0), (int)F, limit, slope, shift, plan.row_pair.data, plan.wts.data, stream));
+  return out;
+}
+
+Tensor Kernels::moe_sum_unweighed(const Tensor& y, const MoePlan& plan) {
+  expect(y, "experts' outputs", dtype_);
+  if (y.shape.size() != 2 || y.dim(0) != plan.row_pair.dim(0)) throw EngineError("experts (sum): outputs " + y.describe());
+  const int64_t T = plan.idx.dim(0), W = y.dim(1);
+  Tensor out = empty({T, W}, DType::F32);
+  call(fn_->moe_combine(out.data, y.data, nullptr, plan.pair_row.data, (int)T, (int)W, plan.top, stream));
+  return out;
+}
+
+// ----------------------------------------------------------------------- attention through a latent
+Tensor Kernels::norm_columns(const Tensor& x, int64_t col, int64_t n, const Tensor& w, float eps, int64_t width) {
+  expect(x, "norm input", dtype_);
+  if (x.shape.size() != 2 || col < 0 || n < 1 || col + n > x.dim(1) || width < n) throw EngineError("norm of columns " + std::to_string(col) + ".. of " + x.describe());
+  const int wf = norm_weight(w, "norm weight", n);
+  Tensor out = empty({x.dim(0), width});
+  call(fn_->norm_columns(out.data, width, x.data, x.dim(1), (int)col, (int)n, w.data, wf, eps, (int)x.dim(0), stream));
+  return out;
+}
+
+void Kernels::gemm_heads(Tensor& out, int64_t out_stride, const Tensor& x, int64_t x_col, int64_t x_stride, const Tensor& w) {
+  expect(out, "heads' outputs", dtype_);
+  expect(x, "heads' inputs", dtype_);
+  expect(w, "heads' weights", dtype_);
+  if (out.shape.size() != 2 || x.shape.size() != 2 || w.shape.size() != 3 || out.dim(0) != x.dim(0) || x_col < 0 || out_stride < 0 || x_stride < 0)
+    throw EngineError("product a head: outputs " + out.describe() + ", inputs " + x.describe() + ", weights " + w.describe());
+  const int64_t H = w.dim(0), N = w.dim(1), K = w.dim(2);
+  const int vec = 16 / dtype_bytes(dtype_);
+  if (x_col + (H - 1) * x_stride + K > x.dim(1) || (H - 1) * out_stride + N > out.dim(1) || x_col % vec)
+    throw EngineError("product a head: " + std::to_string(H) + " heads of " + std::to_string(K) + " -> " + std::to_string(N) + " do not fit inputs " +
+                      x.describe() + " from column " + std::to_string(x_col) + " or outputs " + out.describe());
+  call(fn_->gemm_heads(out.data, out.dim(1), out_stride, static_cast<const char*>(x.data) + (size_t)x_col * dtype_bytes(dtype_), x.dim(1), x_stride, w.data,
+                       (int)x.dim(0), (int)H, (int)N, (int)K, stream));
+}
+
+void Kernels::latent_post(const Tensor& proj, int64_t kv_col, const Tensor& q, int64_t q_stride, int64_t q_first, Tensor& q_abs, const Tensor* k_cache,
+                          const Tensor* v_cache, int page_size, const Tensor* norm_w, float eps, const Tensor& inv_freq, bool neighbours,
+                          const Tensor& positions, const Tensor* slots, int r, int dr) {
+  expect(q, "queries", dtype_);
+  expect(q_abs, "queries as the cache meets them", dtype_);
+  if (q.shape.size() != 2 || q_abs.shape.size() != 3 || q_abs.dim(0) != q.dim(0) || r < 1 || dr < 2 || q_abs.dim(2) < r + dr)
+    throw EngineError("latent attention: queries " + q.describe() + " to " + q_abs.describe());
+  const int64_t T = q.dim(0), H = q_abs.dim(1), D = q_abs.dim(2);
+  if (q_first < 0 || q_stride < q_first + dr || (H - 1) * q_stride + q_first + dr > q.dim(1))
+    throw EngineError("latent attention: " + std::to_string(H) + " heads do not fit queries " + q.describe());
+  expect(inv_freq, "rotation frequencies", DType::F32, {(int64_t)dr / 2});
+  expect(positions, "positions", DType::I32, {T});
+  const bool store = kv_col >= 0;
+  int wf = 0;
+  if (store) {
+    expect(proj, "latent projection", dtype_);
+    if (proj.shape.size() != 2 || proj.dim(0) != T || kv_col + r + dr > proj.dim(1)) throw EngineError("latent attention: the projection is " + proj.describe());
+    if (!k_cache || !v_cache || !slots || !norm_w) throw EngineError("latent attention: a store needs both caches, slots and the norm's weight");
+    if (k_cache->shape.size() != 4) throw EngineError("k cache is " + k_cache->describe());
+    const int64_t pages = k_cache->dim(0);
+    expect(*k_cache, "k cache", dtype_, {pages, 1, page_size, D});
+    expect(*v_cache, "v cache", dtype_, {pages, 1, D, page_size});
+    expect(*slots, "slots", DType::I32, {T});
+    wf = norm_weight(*norm_w, "latent norm weight", r);
+  }
+  call(fn_->latent_post(store ? static_cast<const char*>(proj.data) + (size_t)kv_col * dtype_bytes(dtype_) : nullptr, store ? proj.dim(1) : 0, q.data,
+                        q.dim(1), q_stride, (int)q_first, q_abs.data, store ? k_cache->data : nullptr, store ? v_cache->data : nullptr,
+                        store ? norm_w->data : nullptr, wf, eps, inv_freq.data, neighbours ? 1 : 0, positions.data, store ? slots->data : nullptr, (int)T,
+                        (int)H, r, dr, (int)D, page_size, stream));
+}
+
+Tensor Kernels::qkv_post_norm_angles_paired(const Tensor& qkv, int nq, int nkv, int d, const Tensor* k_cache, const Tensor* v_cache, int page_size,
+                                            const Tensor* q_w, const Tensor* k_w, int norm_d, float eps, const Tensor& inv_freq, float mag,
+                                            bool neighbours, const Tensor& positions, const Tensor* slots) {
+  expect(qkv, "qkv", dtype_);
+  const int64_t W = (int64_t)(nq + 2 * nkv) * d;
+  if (qkv.shape.size() != 2 || qkv.dim(1) < W) throw EngineError("qkv_post: rows are " + qkv.describe() + ", expected a width of at least " + std::to_string(W));
+  const int64_t T = qkv.dim(0);
+  expect(inv_freq, "rotation frequencies", DType::F32);
+  if (norm_d < 1 || norm_d > d || inv_freq.shape.size() != 1 || inv_freq.dim(0) < 1 || 2 * inv_freq.dim(0) > norm_d)
+    throw EngineError("qkv_post: rotation frequencies are " + inv_freq.describe() + " for a head of " + std::to_string(norm_d) + " in " + std::to_string(d));
+  int wf = 0;
+  if (q_w) wf = norm_weight(*q_w, "q norm weight", norm_d);
+  if (k_w) {
+    const int wf2 = norm_weight(*k_w, "k norm weight", norm_d);
+    if (q_w && wf2 != wf) throw EngineError("qkv_post: q and k norm weights must have the same type");
+    wf = wf2;
+  }
+  expect(positions, "positions", DType::I32, {T});
+  Tensor q_out;
+  if (nq) q_out = empty({T, nq, d});
+  if (nkv) {
+    if (!k_cache || !v_cache || !slots) throw EngineError("qkv_post: a store needs both caches and slots");
+    if (k_cache->shape.size() != 4) throw EngineError("k cache is " + k_cache->describe());
+    const int64_t pages = k_cache->dim(0);
+    expect(*k_cache, "k cache", dtype_, {pages, nkv, page_size, d});
+    expect(*v_cache, "v cache", dtype_, {pages, nkv, d, page_size});
+    expect(*slots, "slots", DType::I32, {T});
+  }
+  call(fn_->qkv_post_norm_angles_paired(qkv.data, qkv.dim(1), nq ? q_out.data : nullptr, nkv ? k_cache->data : nullptr, nkv ? v_cache->data : nullptr,
+                                        q_w ? q_w->data : nullptr, k_w ? k_w->data : nullptr, wf, norm_d, eps, inv_freq.data, mag, (int)inv_freq.dim(0),
+                                        neighbours ? 1 : 0, positions.data, nkv ? slots->data : nullptr, (int)T, nq, nkv, d, page_size, stream));
+  return q_out;
+}
+
+Tensor Kernels::linear_rule(const Tensor& x, int64_t q_col, int64_t k_col, int64_t v_col, const Tensor& head_decay, bool silu_inputs, Tensor& state,
+                            const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H, int d, int dv, float q_scale) {
+  expect(x, "linear attention input", dtype_);
+  expect(state, "state", DType::F32);
+  if (x.shape.size() != 2 || state.shape.size() != 2 || q_col < 0 || k_col < 0 || v_col < 0 || std::max(q_col, k_col) + (int64_t)H * d > x.dim(1) ||
+      v_col + (int64_t)H * dv > x.dim(1) || state.dim(1) < (int64_t)H * d * dv)
+    throw EngineError("linear attention: input " + x.describe() + ", state " + state.describe());
+  const int64_t T = x.dim(0), S = slots.numel();
+  expect(head_decay, "the heads' decays", DType::F32, {(int64_t)H});
+  expect(positions, "positions", DType::I32, {T});
+  expect(cu_q, "cu_q", DType::I32, {S + 1});
+  expect(slots, "state slots", DType::I32, {S});
+  Tensor out = empty({T, H, dv}, DType::F32);
+  call(fn_->linear_rule(out.data, x.data, x.dim(1), (int)q_col, (int)k_col, (int)v_col, head_decay.data, silu_inputs ? 1 : 0, state.data, state.dim(1),
+                        cu_q.data, positions.data, slots.data, (int)S, H, d, dv, q_scale, stream));
+  return out;
+}
+
+Tensor Kernels::side_gate(const Tensor& gate, const Tensor& table, const Tensor& ids, int64_t first, int64_t n) {
+  expect(gate, "side gate", dtype_);
+  expect(table, "side table", dtype_);
+  if (gate.shape.size() != 2 || table.shape.size() != 2 || first < 0 || n < 1 || n > gate.dim(1) || first + n > table.dim(1))
+    throw EngineError("token side input: gate " + gate.describe() + ", table " + table.describe());
+  expect(ids, "ids", DType::I32, {gate.dim(0)});
+  Tensor out = empty(gate.shape);
+  call(fn_->side_gate(out.data, gate.dim(1), gate.data, gate.dim(1), table.data, table.dim(1), ids.data, (int)first, (int)n, (int)gate.dim(0), stream));
   return out;
 }
 

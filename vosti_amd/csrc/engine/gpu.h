@@ -109,6 +109,8 @@ class Kernels {
   Tensor swiglu(const Tensor& gate_up);
   Tensor gather_rows(const Tensor& x, const Tensor& rows);
   Tensor to_f32(const Tensor& x);
+  // A 32-bit tensor as elements (the tensor itself where the elements are 32-bit).
+  Tensor to_elements(const Tensor& x);
   // Columns [first, first + count) of a [rows, width] tensor as a tensor of their own.
   Tensor columns(const Tensor& x, int64_t first, int64_t count);
   // dst[:, dst_first : dst_first + count] = src[:, src_first : src_first + count], rows alike.
@@ -228,6 +230,33 @@ class Kernels {
   // block is skipped); [M, N] elements, the bits gemm gives for the same rows and matrix.  K in whole pairs of slabs.
   Tensor gemm_grouped(const Tensor& act, const Tensor& w, const Tensor& block_weights);
   bool gemm_grouped_takes(int64_t K) const;
+  // moe_route with a choice of score: 0 as moe_route; 1: a chosen expert's weight is the logistic function of its logit.
+  MoePlan moe_route_scored(const Tensor& h, const Tensor& router, int top, float weight_eps, int tile_rows, const Tensor* bias, int score_kind);
+  // moe_glu for experts that read their input times the pair's weight: every row's gate and up values are multiplied by
+  // its pair's weight before the clamps; moe_sum_unweighed then adds a token's rows as they are.
+  Tensor moe_glu_weighed(const Tensor& gate_up, float limit, float slope, float shift, const MoePlan& plan);
+  Tensor moe_sum_unweighed(const Tensor& y, const MoePlan& plan);
+  // ---- attention through a latent (latent.hip)
+  // norm(x[:, col : col + n]) * w as elements [T, width], the columns beyond n zero.
+  Tensor norm_columns(const Tensor& x, int64_t col, int64_t n, const Tensor& w, float eps, int64_t width);
+  // out[:, h * out_stride : + N] = x[:, x_col + h * x_stride : + K] W[h]^T for every head; w [H, N, K]; out [T, out_width] elements.
+  void gemm_heads(Tensor& out, int64_t out_stride, const Tensor& x, int64_t x_col, int64_t x_stride, const Tensor& w);
+  // The latent's norm, the rotation of the key part and of the heads' rotated query parts, and the cache store, in one
+  // launch.  q_abs [T, H, D]: its columns [r, D) of every head are written.  kv_col < 0: queries only.
+  void latent_post(const Tensor& proj, int64_t kv_col, const Tensor& q, int64_t q_stride, int64_t q_first, Tensor& q_abs, const Tensor* k_cache,
+                   const Tensor* v_cache, int page_size, const Tensor* norm_w, float eps, const Tensor& inv_freq, bool neighbours,
+                   const Tensor& positions, const Tensor* slots, int r, int dr);
+  // qkv_post_norm_angles with a choice of pairs: neighbours true turns elements 2c and 2c + 1; the norms may be absent.
+  Tensor qkv_post_norm_angles_paired(const Tensor& qkv, int nq, int nkv, int d, const Tensor* k_cache, const Tensor* v_cache, int page_size,
+                                     const Tensor* q_w, const Tensor* k_w, int norm_d, float eps, const Tensor& inv_freq, float mag, bool neighbours,
+                                     const Tensor& positions, const Tensor* slots);
+  // ---- linear attention with one fixed decay a head (delta.hip)
+  // S <- decay[h] S + k v^T, o = S^T q; silu_inputs: q, k and v pass silu first.  decay [H] floats.  Returns o [T, H, dv] floats.
+  Tensor linear_rule(const Tensor& x, int64_t q_col, int64_t k_col, int64_t v_col, const Tensor& head_decay, bool silu_inputs, Tensor& state,
+                     const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H, int d, int dv, float q_scale);
+  // ---- a token's slice of a second embedding table, gated (stream.hip)
+  // gelu(gate[:, 0:n]) * table[ids, first : first + n] as elements [T, gate.dim(1)], zero beyond n.
+  Tensor side_gate(const Tensor& gate, const Tensor& table, const Tensor& ids, int64_t first, int64_t n);
   void relu_square(Tensor& x);                 // x <- max(x, 0)^2
   int segment_keys() const { return segment_keys_; }
   int item_rows() const { return item_rows_; }

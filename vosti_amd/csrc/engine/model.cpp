@@ -331,6 +331,7 @@ std::vector<CacheNeed> DecoderModel::cache_needs() {
 Tensor DecoderModel::forward(const Tensor& ids, StepContext& ctx, std::vector<CacheEntry>& caches, const Tensor& want_rows) {
   if (!loaded_) throw EngineError("the model has no weights yet");
   if (caches.size() != spec_.schedule.size()) throw EngineError("one cache entry per schedule entry is needed");
+  ctx.ids = ids;
   Tensor hidden = embedding_->forward(ids, ctx), residual;
   for (size_t i = 0; i < spec_.schedule.size(); ++i) {
     auto hr = layers_[spec_.schedule[i].layer]->forward(hidden, residual, ctx, caches[i]);

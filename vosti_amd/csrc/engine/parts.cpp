@@ -83,6 +83,9 @@ std::pair<Tensor, Tensor> PositionEncoding::apply(const Tensor& q, const Tensor&
   auto rotate = [&](const Tensor& x) {
     if (x.shape.size() != 3) throw EngineError("position encoding of " + x.describe() + ", expected [tokens, heads, head size]");
     const int64_t T = x.dim(0), n = x.dim(1), d = x.dim(2);
+    if (freq && pairs_neighbours())
+      return kernels.qkv_post_norm_angles_paired(x.view({T, n * d}), (int)n, 0, (int)d, nullptr, nullptr, 0, nullptr, nullptr, (int)d, 0.f, *freq, magnitude(),
+                                                 true, positions, nullptr);
     if (freq) return kernels.qkv_post_angles(x.view({T, n * d}), (int)n, 0, (int)d, nullptr, nullptr, 0, *freq, magnitude(), positions, nullptr);
     return kernels.qkv_post(x.view({T, n * d}), (int)n, 0, (int)d, nullptr, nullptr, 0, nullptr, nullptr, 0.f, cos, sin, &positions, nullptr);
   };
@@ -333,24 +336,33 @@ class Rotary : public PositionEncoding {
 
 // The same half-rotation with angles that are computed where they are used, in 32-bit, and frequencies whose long
 // wavelengths are stretched (rotary_stretched_frequencies has the rule): numbers rotary_dim, theta and, for a stretch,
-// factor, original, fast, slow.  Cosine and sine are multiplied by 0.1 ln(factor) + 1.
+// factor, original, fast, slow.  Cosine and sine are multiplied by 0.1 ln(factor) + 1.  linear_factor instead of factor:
+// every frequency is divided by it and nothing else changes (rotary_linear_frequencies).  neighbours 1: a pair is a head's
+// elements 2c and 2c + 1 instead of c and c + half.
 class RotaryStretched : public PositionEncoding {
  public:
   RotaryStretched(const PartSpec& s, Kernels& k) : PositionEncoding(k), head_dim_(s.integer("head_dim")), rotary_dim_(s.integer("rotary_dim")) {
     if (rotary_dim_ % 2 || rotary_dim_ <= 0 || rotary_dim_ > head_dim_)
       throw ConfigError("rotary width " + std::to_string(rotary_dim_) + " must be even and at most the head size " + std::to_string(head_dim_));
     std::vector<float> f((size_t)rotary_dim_ / 2);
-    mag_ = rotary_stretched_frequencies(s.number("theta"), (int)rotary_dim_, s.number("factor", 0.0), s.number("original", 1.0), s.number("fast", 1.0),
-                                        s.number("slow", 1.0), f.data());
+    neighbours_ = s.integer("neighbours", 0) != 0;
+    const double linear = s.number("linear_factor", 0.0);
+    if (linear < 0 || (linear > 0 && s.number("factor", 0.0) > 0)) throw ConfigError("a rotation is stretched by 'factor' or by 'linear_factor', not both");
+    if (linear > 0) rotary_linear_frequencies(s.number("theta"), (int)rotary_dim_, linear, f.data());
+    else
+      mag_ = rotary_stretched_frequencies(s.number("theta"), (int)rotary_dim_, s.number("factor", 0.0), s.number("original", 1.0), s.number("fast", 1.0),
+                                          s.number("slow", 1.0), f.data());
     freq_ = zero_weight({rotary_dim_ / 2}, DType::F32);
     hip_check(hipMemcpy(freq_.data, f.data(), f.size() * sizeof(float), hipMemcpyHostToDevice), "rotation frequencies");
   }
   const Tensor* angle_frequencies() override { return &freq_; }
   float magnitude() override { return mag_; }
+  bool pairs_neighbours() const override { return neighbours_; }
 
  private:
   int64_t head_dim_, rotary_dim_;
   float mag_ = 1.f;
+  bool neighbours_ = false;
   Tensor freq_;
 };
 
@@ -360,6 +372,34 @@ struct AttentionItems {
   HostArray prefill, decode;
   int decode_bound = 0, nseg = 0;
 };
+
+// The items of a step, derived once a step and shared by every mixer that runs the paged attention kernels.
+AttentionItems& attention_items(Kernels& kernels, HostStep& step) {
+  auto it = step.memo.find("attention.items");
+  if (it != step.memo.end()) return *static_cast<AttentionItems*>(it->second.get());
+  auto m = std::make_shared<AttentionItems>();
+  const int rows = kernels.item_rows();
+  int decode_keys = 0;
+  for (size_t s = 0; s < step.q_lens.size(); ++s) {
+    if (step.q_lens[s] == 1) {
+      m->decode.data.push_back((int32_t)s);
+      m->decode.data.push_back(0);
+      decode_keys = std::max(decode_keys, step.k_lens[s]);
+    } else {
+      for (int off = 0; off < step.q_lens[s]; off += rows) {
+        m->prefill.data.push_back((int32_t)s);
+        m->prefill.data.push_back(off);
+      }
+    }
+  }
+  m->prefill.shape = {(int64_t)m->prefill.data.size() / 2, 2};
+  m->decode.shape = {(int64_t)m->decode.data.size() / 2, 2};
+  // Recorded launches must cover every length that the tables can hold.
+  m->decode_bound = step.frozen ? step.k_len_bound : decode_keys;
+  m->nseg = (m->decode_bound + kernels.segment_keys() - 1) / kernels.segment_keys();
+  step.memo["attention.items"] = m;
+  return *m;
+}
 
 // Causal grouped-query attention over the paged cache (src/exec/dense_swiglu_decoder.rs:171-367): QKV
 // projection without bias, per-head norm of q and k, rotary encoding, store of k and v, attention, output
@@ -472,32 +512,7 @@ class Attention : public Mixer {
   }
   const char* step_inputs_key() const override { return "attention.items"; }
 
-  AttentionItems& items(HostStep& step) {
-    auto it = step.memo.find("attention.items");
-    if (it != step.memo.end()) return *static_cast<AttentionItems*>(it->second.get());
-    auto m = std::make_shared<AttentionItems>();
-    const int rows = kernels.item_rows();
-    int decode_keys = 0;
-    for (size_t s = 0; s < step.q_lens.size(); ++s) {
-      if (step.q_lens[s] == 1) {
-        m->decode.data.push_back((int32_t)s);
-        m->decode.data.push_back(0);
-        decode_keys = std::max(decode_keys, step.k_lens[s]);
-      } else {
-        for (int off = 0; off < step.q_lens[s]; off += rows) {
-          m->prefill.data.push_back((int32_t)s);
-          m->prefill.data.push_back(off);
-        }
-      }
-    }
-    m->prefill.shape = {(int64_t)m->prefill.data.size() / 2, 2};
-    m->decode.shape = {(int64_t)m->decode.data.size() / 2, 2};
-    // Recorded launches must cover every length that the tables can hold.
-    m->decode_bound = step.frozen ? step.k_len_bound : decode_keys;
-    m->nseg = (m->decode_bound + kernels.segment_keys() - 1) / kernels.segment_keys();
-    step.memo["attention.items"] = m;
-    return *m;
-  }
+  AttentionItems& items(HostStep& step) { return attention_items(kernels, step); }
   void step_inputs(HostStep& step, std::vector<std::pair<std::string, HostArray>>& out) override {
     AttentionItems& m = items(step);
     out.emplace_back("attention.prefill_items", m.prefill);
@@ -545,9 +560,12 @@ class Attention : public Mixer {
     Tensor q;
     if (norm_angles) {
       const Norm* en = q_norm_ ? q_norm_.get() : k_norm_.get();
-      q = k.qkv_post_norm_angles(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size,
-                                 q_norm_ ? q_norm_->row_scale_weight() : nullptr, k_norm_ && cache.writable ? k_norm_->row_scale_weight() : nullptr, dk_,
-                                 en->eps(), *position_->angle_frequencies(), position_->magnitude(), ctx.positions, &tables.slots);
+      q = k.qkv_post_norm_angles_paired(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size,
+                                        q_norm_ ? q_norm_->row_scale_weight() : nullptr, k_norm_ && cache.writable ? k_norm_->row_scale_weight() : nullptr,
+                                        dk_, en->eps(), *position_->angle_frequencies(), position_->magnitude(), position_->pairs_neighbours(),
+                                        ctx.positions, &tables.slots);
+    } else if (position_ && position_->pairs_neighbours()) {
+      throw ConfigError("attention: a rotation of neighbouring pairs is built together with head norms");
     } else if (bias_) {
       const int64_t bw = (int64_t)(nq_ + (cache.writable ? 2 * nkv_ : 0)) * d_;
       q = k.qkv_post_bias(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size, &tables.slots, b_qkv_.rows(0, bw));
@@ -1131,14 +1149,19 @@ class PairMean : public Mixer {
 // weight_eps 0 the weights are then the softmax over the chosen logits alone), gated (an expert is
 // W_down (g * sigmoid(glu_slope * g) * (u + up_shift)) with g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit)),
 // shared_size (> 0: one more expert of that inner size and the same form, with shared_limit, that every token uses
-// with weight 1; its output is added to the sum).
+// with weight 1; its output is added to the sum), score (1: the weights are the logistic function of the chosen logits, not
+// divided by anything), weigh_input (1: the output is the sum of expert(weight * h); since W (w h) = w (W h), the weight
+// multiplies the gate and up outputs before their clamps, and the sum adds the experts' outputs as they are).
 class RoutedExperts : public FeedForward {
  public:
   RoutedExperts(const PartSpec& s, Kernels& k)
       : FeedForward(k), hidden_(s.integer("hidden_size")), inter_(s.integer("intermediate_size")), experts_((int)s.integer("experts")),
         top_((int)s.integer("top")), weight_eps_((float)s.number("weight_eps", 0.0)), bias_(s.integer("router_bias", 0) != 0),
         gated_(s.integer("gated", 0) != 0), limit_((float)s.number("limit", 0.0)), slope_((float)s.number("glu_slope", 1.0)),
-        shift_((float)s.number("up_shift", 0.0)), shared_(s.integer("shared_size", 0)), shared_limit_((float)s.number("shared_limit", 0.0)) {
+        shift_((float)s.number("up_shift", 0.0)), shared_(s.integer("shared_size", 0)), shared_limit_((float)s.number("shared_limit", 0.0)),
+        score_((int)s.integer("score", 0)), weigh_input_(s.integer("weigh_input", 0) != 0) {
+    if (score_ < 0 || score_ > 1) throw ConfigError("experts: 'score' is 0 (softmax) or 1 (the logistic function of a chosen logit)");
+    if (weigh_input_ && (!gated_ || shared_ > 0)) throw ConfigError("experts whose weights scale their inputs are built in the gated form, without a shared expert");
     if (experts_ < 1 || top_ < 1 || top_ > experts_) throw ConfigError("a mixture of " + std::to_string(experts_) + " experts cannot choose " + std::to_string(top_));
     if (gated_ && !(limit_ > 0.f)) throw ConfigError("gated experts need a positive 'limit'");
     if (shared_ < 0 || (shared_ > 0 && (!gated_ || !(shared_limit_ > 0.f))))
@@ -1194,12 +1217,15 @@ class RoutedExperts : public FeedForward {
     // the rows are sorted by expert into blocks of 128 and go through the engine's tile product, every block with its
     // expert's matrix.  Both are launched from numbers on the GPU alone and give the same bits.
     if (pairs < (int64_t)kRowsAnExpertForTiles * experts_ || !k.gemm_grouped_takes(hidden_) || !k.gemm_grouped_takes(w_down_.dim(2))) {
-      const Kernels::MoePlan plan = k.moe_route(x, router_, top_, weight_eps_, 16, bias);
+      const Kernels::MoePlan plan = k.moe_route_scored(x, router_, top_, weight_eps_, 16, bias, score_);
+      if (weigh_input_)
+        return k.moe_sum_unweighed(k.moe_down(k.moe_glu_weighed(k.moe_up_plain(x, w_up_, plan), limit_, slope_, shift_, plan), w_down_, plan), plan);
       const Tensor act = gated_ ? k.moe_glu(k.moe_up_plain(x, w_up_, plan), limit_, slope_, shift_) : k.moe_up(x, w_up_, plan);
       return k.moe_sum(k.moe_down(act, w_down_, plan), plan, extra);
     }
-    const Kernels::MoePlan plan = k.moe_route(x, router_, top_, weight_eps_, 128, bias);
+    const Kernels::MoePlan plan = k.moe_route_scored(x, router_, top_, weight_eps_, 128, bias, score_);
     Tensor act = k.gemm_grouped(k.gather_rows(x, plan.row_token), w_up_, plan.tile_expert);
+    if (weigh_input_) return k.moe_sum_unweighed(k.gemm_grouped(k.moe_glu_weighed(act, limit_, slope_, shift_, plan), w_down_, plan.tile_expert), plan);
     if (gated_) act = k.moe_glu(act, limit_, slope_, shift_);
     else k.relu_square(act);
     return k.moe_sum(k.gemm_grouped(act, w_down_, plan.tile_expert), plan, extra);
@@ -1214,6 +1240,8 @@ class RoutedExperts : public FeedForward {
   float limit_, slope_, shift_;
   int64_t shared_;
   float shared_limit_;
+  int score_;              // 0: softmax scores; 1: a chosen expert's weight is the logistic function of its logit
+  bool weigh_input_;       // a weight scales what its expert reads (the gate and up outputs before their clamps), not what it gives
   Tensor router_, router_bias_, w_up_, w_down_, w_shared_in_, w_shared_down_;
 };
 
@@ -1259,6 +1287,303 @@ class ParallelSumBlock : public Block {
   bool has_ffn_ = true;
 };
 
+// A weight laid out anew on the host: element (i, j) of the result [rows, cols] is the source's element from(i, j), or zero
+// where that gives a negative row.  For arrangements that a strided copy cannot express (a transpose a head, say).
+Tensor rearranged(const Tensor& w, int64_t rows, int64_t cols, const std::function<std::pair<int64_t, int64_t>(int64_t, int64_t)>& from) {
+  if (w.shape.size() != 2) throw EngineError("a weight of " + w.describe() + " cannot be rearranged as a matrix");
+  const size_t e = (size_t)dtype_bytes(w.dtype);
+  std::vector<char> src(w.bytes()), dst((size_t)(rows * cols) * e, 0);
+  if (w.numel()) hip_check(hipMemcpy(src.data(), w.data, w.bytes(), hipMemcpyDeviceToHost), "reading a weight back");
+  for (int64_t i = 0; i < rows; ++i)
+    for (int64_t j = 0; j < cols; ++j) {
+      const auto ij = from(i, j);
+      if (ij.first < 0) continue;
+      if (ij.first >= w.dim(0) || ij.second < 0 || ij.second >= w.dim(1)) throw EngineError("a weight's rearrangement reads outside " + w.describe());
+      std::copy_n(src.data() + (size_t)(ij.first * w.dim(1) + ij.second) * e, e, dst.data() + (size_t)(i * cols + j) * e);
+    }
+  Tensor out = zero_weight({rows, cols}, w.dtype);
+  if (out.numel()) hip_check(hipMemcpy(out.data, dst.data(), dst.size(), hipMemcpyHostToDevice), "writing a weight");
+  return out;
+}
+
+// Attention through a latent.  For the mixer's input h, with H heads, per head d entries that are not rotated and dr that
+// are, value size dv, latent size r and query latent size rq:
+//   c_q = norm(W_dq h) (weight dq.norm), q = W_uq c_q, head by head [d | dr];  W_dkv h = [latent: r | key part: dr];
+//   c = norm(latent) (weight dkv.norm); the key part is rotated by the position and serves every head;
+//   head j: k_j = W_uk[j] c, v_j = W_uv[j] c; score = (q_flat . k_j + rotate(q_rot) . rotated key part) * scale;
+//   softmax over the keys so far; the heads side by side times sigmoid(W_g h); then W_o.
+// Only c and the rotated key part are kept: the cache has one kv head whose key row is [c | rotated part | 0] and whose
+// value row is [c | 0], D = r + dr rounded up to 16 entries.  Since q_flat . (W_uk[j] c) = (W_uk[j]^T q_flat) . c, head j's
+// query meets the cache as [W_uk[j]^T q_flat | rotate(q_rot) | 0], and its output is W_uv[j] times the weighted sum of the
+// cached c: two products a head (gemm_heads) around the engine's paged attention kernels, whose weights are 32-bit.
+// own_kv 0: the layer has no W_dkv and reads the cache of an earlier layer of the same latent and rotation, with W_uk,
+// W_uv, queries and everything else of its own.  Sizes that are no whole 16-byte vectors are padded with zeros in the
+// weights at load.
+class LatentAttention : public Mixer {
+ public:
+  LatentAttention(const PartSpec& s, Kernels& k)
+      : Mixer(k), hidden_(s.integer("hidden_size")), H_((int)s.integer("num_heads")), d_((int)s.integer("head_dim")), dr_((int)s.integer("rotary_dim")),
+        dv_((int)s.integer("value_dim")), r_((int)s.integer("kv_rank")), rq_((int)s.integer("q_rank")), scale_((float)s.number("scale")),
+        eps_((float)s.number("eps")), own_kv_(s.integer("own_kv", 1) != 0), gate_(s.integer("output_gate", 0) != 0) {
+    D_ = (int)round_up((int64_t)r_ + dr_, 16);
+    if (H_ < 1 || d_ < 1 || dr_ < 2 || dr_ % 2 || dv_ < 1 || r_ < 1 || rq_ < 1) throw ConfigError("latent attention: bad sizes");
+    if (D_ > 256) throw ConfigError("latent attention: a latent of " + std::to_string(r_) + " with " + std::to_string(dr_) + " rotated entries: the attention kernels take up to 256 together");
+    const PartSpec* p = s.part("position");
+    if (!p) throw ConfigError("latent attention needs the part 'position'");
+    position_ = build_part<PositionEncoding>("position", *p, k);
+    dp_ = round_up(d_, 8);
+    qs_ = dp_ + round_up(dr_, 8);
+    rqp_ = round_up(rq_, 8);
+    kvp_ = round_up((int64_t)r_ + dr_, 8);
+    dvp_ = round_up(dv_, 8);
+  }
+  std::vector<ParamDecl> params() const override {
+    ParamDecl qn{"q_down_norm.weight", {(int64_t)rq_}, true, true, 0.9, 1.1}, kn{"kv_down_norm.weight", {(int64_t)r_}, true, true, 0.9, 1.1};
+    ParamDecl uq{"q_up.weight", {(int64_t)H_ * (d_ + dr_), (int64_t)rq_}}, uk{"k_up.weight", {(int64_t)H_ * d_, (int64_t)r_}},
+        uv{"v_up.weight", {(int64_t)H_ * dv_, (int64_t)r_}};
+    uq.p0 = uk.p0 = uv.p0 = 0.06;
+    std::vector<ParamDecl> p = {{"q_down.weight", {(int64_t)rq_, hidden_}}, qn, uq, uk, uv, {"o_proj.weight", {hidden_, (int64_t)H_ * dv_}}};
+    if (own_kv_) {
+      p.push_back({"kv_down.weight", {(int64_t)r_ + dr_, hidden_}});
+      p.push_back(kn);
+    }
+    if (gate_) p.push_back({"gate_proj.weight", {(int64_t)H_ * dv_, hidden_}});
+    return p;
+  }
+  std::vector<std::pair<std::string, Part*>> children() override { return {{"position", position_.get()}}; }
+  void load(std::map<std::string, Tensor>& t) override {
+    if (!position_->angle_frequencies()) throw ConfigError("latent attention is built for rotations by computed angles");
+    // One launch projects the query's latent, the latent with its key part (where the layer has them) and the gate.
+    std::vector<Tensor> rows = {pad_matrix(need(t, "q_down.weight"), rqp_, hidden_)};
+    if (own_kv_) rows.push_back(pad_matrix(need(t, "kv_down.weight"), kvp_, hidden_));
+    if (gate_) rows.push_back(pad_row_blocks(need(t, "gate_proj.weight"), H_, dv_, dvp_));
+    w_in_ = rows.size() > 1 ? stack_rows(rows) : rows[0];
+    kv_col_ = own_kv_ ? rqp_ : -1;
+    gate_col_ = rqp_ + (own_kv_ ? kvp_ : 0);
+    q_norm_ = need(t, "q_down_norm.weight");
+    if (own_kv_) kv_norm_ = need(t, "kv_down_norm.weight");
+    const int64_t d = d_, dr = dr_, dp = dp_, qs = qs_, r = r_, dv = dv_, D = D_;
+    // A head's query rows as [d | zeros to dp | dr | zeros to qs], the columns padded to the padded latent.
+    w_uq_ = rearranged(need(t, "q_up.weight"), (int64_t)H_ * qs, rqp_, [=](int64_t i, int64_t j) -> std::pair<int64_t, int64_t> {
+      const int64_t h = i / qs, e = i % qs;
+      if (j >= rq_) return {-1, 0};
+      if (e < d) return {h * (d + dr) + e, j};
+      if (e >= dp && e < dp + dr) return {h * (d + dr) + d + (e - dp), j};
+      return {-1, 0};
+    });
+    // Head h's W_uk transposed: [r, dp], so that a product a head takes q_flat to the latent's side.
+    w_absorb_ = rearranged(need(t, "k_up.weight"), (int64_t)H_ * r, dp, [=](int64_t i, int64_t j) -> std::pair<int64_t, int64_t> {
+                  if (j >= d) return {-1, 0};
+                  return {(i / r) * d + j, i % r};
+                }).view({(int64_t)H_, r, dp});
+    // Head h's W_uv over a whole cache row: [dvp, D], zero where the row holds no latent.
+    const int64_t dvp = dvp_;
+    w_expand_ = rearranged(need(t, "v_up.weight"), (int64_t)H_ * dvp, D, [=](int64_t i, int64_t j) -> std::pair<int64_t, int64_t> {
+                  const int64_t h = i / dvp, n = i % dvp;
+                  if (n >= dv || j >= r) return {-1, 0};
+                  return {h * dv + n, j};
+                }).view({(int64_t)H_, dvp, D});
+    w_o_ = pad_column_blocks(need(t, "o_proj.weight"), H_, dv_, dvp_);
+  }
+  CacheNeed cache_need() const override {
+    CacheNeed n;
+    n.kind = CacheNeed::Pages;
+    n.num_kv_heads = 1;
+    n.head_dim = D_;
+    return n;
+  }
+  const char* step_inputs_key() const override { return "attention.items"; }
+  void step_inputs(HostStep& step, std::vector<std::pair<std::string, HostArray>>& out) override {
+    AttentionItems& m = attention_items(kernels, step);
+    out.emplace_back("attention.prefill_items", m.prefill);
+    out.emplace_back("attention.decode_items", m.decode);
+  }
+  int64_t workspace_floats(HostStep& step) override {
+    AttentionItems& m = attention_items(kernels, step);
+    return m.decode.shape[0] ? kernels.attn_scratch_floats((int)m.decode.shape[0], H_, D_, m.nseg) : 0;
+  }
+  Tensor forward(const Tensor& x, StepContext& ctx, CacheEntry& cache) override {
+    if (cache.kind != CacheNeed::Pages) throw EngineError("latent attention was handed a cache entry without pages");
+    if (cache.writable != own_kv_) throw EngineError("latent attention: a layer writes the cache if and only if it has a latent projection of its own");
+    Kernels& k = kernels;
+    const int64_t T = x.dim(0);
+    GroupTables& tables = ctx.groups.at(cache.group);
+    const Tensor proj = k.gemm(x, w_in_);
+    const Tensor q = k.gemm(k.norm_columns(proj, 0, rq_, q_norm_, eps_, rqp_), w_uq_);
+    Tensor q_abs = k.empty({T, (int64_t)H_, (int64_t)D_});
+    Tensor q_abs_rows = q_abs.view({T, (int64_t)H_ * D_});
+    k.gemm_heads(q_abs_rows, D_, q, 0, qs_, w_absorb_);
+    k.latent_post(proj, kv_col_, q, qs_, dp_, q_abs, &cache.k, &cache.v, cache.page_size, own_kv_ ? &kv_norm_ : nullptr, eps_,
+                  *position_->angle_frequencies(), position_->pairs_neighbours(), ctx.positions, &tables.slots, r_, dr_);
+    Tensor out = k.empty(q_abs.shape);
+    AttentionItems& m = attention_items(k, *ctx.host);
+    const Tensor& prefill_items = ctx.inputs.at("attention.prefill_items");
+    const Tensor& decode_items = ctx.inputs.at("attention.decode_items");
+    if (prefill_items.dim(0))
+      k.paged_attention_capped(out, q_abs, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, prefill_items, 0, scale_, 0, 0, 0.f, nullptr,
+                               ctx.host->k_len_bound, 0, nullptr, 0);
+    if (decode_items.dim(0)) {
+      const Tensor scratch = ctx.workspace(k.attn_scratch_floats((int)decode_items.dim(0), H_, D_, m.nseg));
+      k.paged_attention_capped(out, q_abs, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, decode_items, 1, scale_, 0, 0, 0.f, nullptr,
+                               m.decode_bound, m.nseg, &scratch, 0);
+    }
+    Tensor heads = k.empty({T, (int64_t)H_ * dvp_});
+    k.gemm_heads(heads, dvp_, out.view({T, (int64_t)H_ * D_}), 0, D_, w_expand_);
+    if (gate_) k.gate_mul(heads, proj, gate_col_, 0);
+    return k.gemm(heads, w_o_);
+  }
+
+ private:
+  int64_t hidden_;
+  int H_, d_, dr_, dv_, r_, rq_, D_ = 0;       // D_: the head size of the cache and the attention kernels
+  float scale_, eps_;
+  bool own_kv_, gate_;
+  int64_t dp_ = 0, qs_ = 0, rqp_ = 0, kvp_ = 0, dvp_ = 0, kv_col_ = -1, gate_col_ = 0;
+  std::unique_ptr<PositionEncoding> position_;
+  Tensor w_in_, w_uq_, w_absorb_, w_expand_, w_o_, q_norm_, kv_norm_;
+};
+
+// Linear attention with one fixed decay a head.  For the mixer's input h:
+//   q = silu(W_q h), k = silu(W_k h) (heads x key size), v = silu(W_v h) (heads x value size);
+//   per head, token by token:  S <- decay[head] S + k v^T;  o = S^T q  (no other scale);
+//   y = norm(the heads' o side by side) (one root mean square over all of them, a weight of that width) * sigmoid(W_g h);
+//   out = W_o y.
+// A request's state slot holds the heads' S in 32-bit, zero at the request's start.  The four input projections are one
+// launch; the recurrence is the delta rule's walk without its correction term, with the decays of the heads (numbers
+// decay.0, decay.1, ...) in place of decays per token and channel; the read-out's norm and gate are one launch.
+class FixedDecayAttention : public Mixer {
+ public:
+  FixedDecayAttention(const PartSpec& s, Kernels& k)
+      : Mixer(k), hidden_(s.integer("hidden_size")), H_((int)s.integer("num_heads")), d_((int)s.integer("key_dim")), dv_((int)s.integer("value_dim")),
+        eps_((float)s.number("eps")) {
+    if (H_ < 1 || d_ < 1 || dv_ < 1 || d_ > 1024) throw ConfigError("linear attention: heads of " + std::to_string(d_) + " x " + std::to_string(dv_));
+    std::vector<float> decay((size_t)H_);
+    for (int h = 0; h < H_; ++h) decay[h] = (float)s.number("decay." + std::to_string(h));
+    decay_ = zero_weight({(int64_t)H_}, DType::F32);
+    hip_check(hipMemcpy(decay_.data, decay.data(), decay.size() * sizeof(float), hipMemcpyHostToDevice), "the heads' decays");
+    qk_ = round_up((int64_t)H_ * d_, 8);
+    v_ = round_up((int64_t)H_ * dv_, 8);
+  }
+  std::vector<ParamDecl> params() const override {
+    const int64_t hd = (int64_t)H_ * d_, hv = (int64_t)H_ * dv_;
+    ParamDecl q{"q_proj.weight", {hd, hidden_}}, kk{"k_proj.weight", {hd, hidden_}}, vv{"v_proj.weight", {hv, hidden_}};
+    q.p0 = kk.p0 = vv.p0 = 0.1;
+    ParamDecl norm{"out_norm.weight", {hv}, true, true, 0.9, 1.1};
+    return {q, kk, vv, {"gate_proj.weight", {hv, hidden_}}, norm, {"o_proj.weight", {hidden_, hv}}};
+  }
+  void load(std::map<std::string, Tensor>& t) override {
+    w_in_ = stack_rows({pad_matrix(need(t, "q_proj.weight"), qk_, hidden_), pad_matrix(need(t, "k_proj.weight"), qk_, hidden_),
+                        pad_matrix(need(t, "v_proj.weight"), v_, hidden_), pad_matrix(need(t, "gate_proj.weight"), v_, hidden_)});
+    out_norm_ = need(t, "out_norm.weight");
+    w_o_ = pad_matrix(need(t, "o_proj.weight"), hidden_, v_);      // the read-out's width as whole 16-byte vectors
+  }
+  CacheNeed cache_need() const override {
+    CacheNeed n;
+    n.kind = CacheNeed::State;
+    n.state_shape = {(int64_t)H_ * d_ * dv_};
+    n.state_dtype = DType::F32;
+    return n;
+  }
+  Tensor forward(const Tensor& x, StepContext& ctx, CacheEntry& cache) override {
+    if (cache.kind != CacheNeed::State) throw EngineError("linear attention was handed a cache entry without state");
+    Kernels& k = kernels;
+    const Tensor proj = k.gemm(x, w_in_);
+    const Tensor o = k.linear_rule(proj, 0, qk_, 2 * qk_, decay_, true, cache.state, ctx.cu_q, ctx.positions, ctx.state_slots, H_, d_, dv_, 1.f);
+    // One norm over all heads: the read-out as one head of H * dv entries.
+    const Tensor all = o.view({o.dim(0), 1, (int64_t)H_ * dv_});
+    return k.gemm(k.gated_head_norm(all, proj, 2 * qk_ + v_, out_norm_, 1, H_ * dv_, eps_, 0, v_), w_o_);
+  }
+
+ private:
+  int64_t hidden_;
+  int H_, d_, dv_;
+  float eps_;
+  int64_t qk_ = 0, v_ = 0;
+  Tensor w_in_, w_o_, out_norm_, decay_;
+};
+
+// What a layer adds from the token's own second embedding: with e the columns [first, first + n) of table[token],
+//   g = gelu(W_gate x) * e;  y = W_out g;  the layer's norm 'side_out' then adds norm(y) to the stream.
+// The table is one tensor for all layers that use it; n that is no whole 16-byte vector is padded with zeros in the weights.
+class TokenSide : public Part {
+ public:
+  TokenSide(Kernels& k, int64_t hidden, int64_t vocab, int64_t n, int64_t first, int64_t table_width)
+      : Part(k), hidden_(hidden), vocab_(vocab), n_(n), first_(first), width_(table_width) {
+    if (n_ < 1 || first_ < 0 || first_ + n_ > width_) throw ConfigError("a token side input of " + std::to_string(n_) + " columns from " + std::to_string(first_) + " of " + std::to_string(width_));
+  }
+  std::vector<ParamDecl> params() const override {
+    ParamDecl table{"table", {vocab_, width_}}, gate{"gate_proj.weight", {n_, hidden_}}, out{"out_proj.weight", {hidden_, n_}};
+    table.p0 = 1.0;
+    gate.p0 = 0.05;
+    out.p0 = 0.2;
+    return {table, gate, out};
+  }
+  void load(std::map<std::string, Tensor>& t) override {
+    table_ = need(t, "table");
+    const int64_t np = round_up(n_, 8);
+    w_gate_ = pad_matrix(need(t, "gate_proj.weight"), np, hidden_);
+    w_out_ = pad_matrix(need(t, "out_proj.weight"), hidden_, np);
+  }
+  // x: the stream as elements.
+  Tensor forward(const Tensor& x, StepContext& ctx) {
+    return kernels.gemm(kernels.side_gate(kernels.gemm(x, w_gate_), table_, ctx.ids, first_, n_), w_out_);
+  }
+
+ private:
+  int64_t hidden_, vocab_, n_, first_, width_;
+  Tensor table_, w_gate_, w_out_;
+};
+
+// A residual stream x in 32-bit whose sublayers read it as it is (rounded to elements), with a norm on their outputs only:
+//   x <- x + norm_mixer_out(mixer(x));  x <- x + norm_ffn_out(ffn(x)) (if the layer has a feed-forward);
+//   x <- x + norm_side_out(side(x, token)) (if the numbers side_dim, side_first, side_width and vocab_size are given:
+//   TokenSide above).
+class PostNormBlock : public Block {
+ public:
+  PostNormBlock(Kernels& k, std::unique_ptr<Mixer> mixer, std::unique_ptr<FeedForward> ffn, std::map<std::string, std::unique_ptr<Norm>> norms,
+                const std::map<std::string, double>& numbers)
+      : Block(k), mixer_(std::move(mixer)), ffn_(std::move(ffn)), norms_(std::move(norms)) {
+    auto number = [&](const char* name) {
+      auto it = numbers.find(name);
+      if (it == numbers.end()) throw ConfigError(std::string("a post_norm block needs the number '") + name + "'");
+      return (int64_t)it->second;
+    };
+    hidden_ = number("hidden_size");
+    has_ffn_ = dynamic_cast<NoFeedForward*>(ffn_.get()) == nullptr;
+    if (!norms_.count("mixer_out")) throw ConfigError("a post_norm block needs the norm 'mixer_out'");
+    if (has_ffn_ && !norms_.count("ffn_out")) throw ConfigError("a post_norm block with a feed-forward needs the norm 'ffn_out'");
+    if (numbers.count("side_dim")) {
+      if (!norms_.count("side_out")) throw ConfigError("a post_norm block with a token side input needs the norm 'side_out'");
+      side_.reset(new TokenSide(k, hidden_, number("vocab_size"), number("side_dim"), number("side_first"), number("side_width")));
+    }
+  }
+  std::vector<std::pair<std::string, Part*>> children() override {
+    std::vector<std::pair<std::string, Part*>> c = {{"mixer", mixer_.get()}, {"feed_forward", ffn_.get()}};
+    for (auto& n : norms_) c.emplace_back("norms." + n.first, n.second.get());
+    if (side_) c.emplace_back("side", side_.get());
+    return c;
+  }
+  Mixer& mixer() override { return *mixer_; }
+  std::pair<Tensor, Tensor> forward(const Tensor& hidden, Tensor residual, StepContext& ctx, CacheEntry& cache) override {
+    Kernels& k = kernels;
+    if (hidden.dtype != DType::F32 || hidden.shape.size() != 2 || hidden.dim(1) != hidden_)
+      throw EngineError("a post_norm block takes the 32-bit residual stream, not " + hidden.describe());
+    Tensor stream = hidden;
+    norms_["mixer_out"]->forward_scaled_add(mixer_->forward(k.to_elements(stream), ctx, cache), stream, stream, 1.f);
+    if (has_ffn_) norms_["ffn_out"]->forward_scaled_add(ffn_->forward(k.to_elements(stream), ctx), stream, stream, 1.f);
+    if (side_) norms_["side_out"]->forward_scaled_add(side_->forward(k.to_elements(stream), ctx), stream, stream, 1.f);
+    return {stream, residual};
+  }
+
+ private:
+  std::unique_ptr<Mixer> mixer_;
+  std::unique_ptr<FeedForward> ffn_;
+  std::map<std::string, std::unique_ptr<Norm>> norms_;
+  std::unique_ptr<TokenSide> side_;
+  int64_t hidden_ = 0;
+  bool has_ffn_ = true;
+};
+
 template <class T>
 PartFactory factory() {
   return [](const PartSpec& s, Kernels& k) { return std::unique_ptr<Part>(new T(s, k)); };
@@ -1293,6 +1618,12 @@ void register_standard_parts() {
     register_block("parallel_sum", [](Kernels& k, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
                                       std::map<std::string, std::unique_ptr<Norm>> n, const std::map<std::string, double>& numbers) {
       return std::unique_ptr<Block>(new ParallelSumBlock(k, std::move(m), std::move(f), std::move(n), numbers));
+    });
+    register_part("mixer", "latent_attention", factory<LatentAttention>());
+    register_part("mixer", "fixed_decay_attention", factory<FixedDecayAttention>());
+    register_block("post_norm", [](Kernels& k, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
+                                   std::map<std::string, std::unique_ptr<Norm>> n, const std::map<std::string, double>& numbers) {
+      return std::unique_ptr<Block>(new PostNormBlock(k, std::move(m), std::move(f), std::move(n), numbers));
     });
     register_part("norm", "rmsnorm", factory<RMSNorm>());
     register_part("position", "rotary", factory<Rotary>());

@@ -50,7 +50,7 @@ struct GroupTables {
 struct StepContext {
   Kernels* kernels = nullptr;
   int num_tokens = 0, num_seqs = 0;
-  Tensor positions, cu_q, k_len, state_slots;
+  Tensor ids, positions, cu_q, k_len, state_slots;   // ids: the step's tokens, for parts that look a token up a second time
   std::vector<GroupTables> groups;
   HostStep* host = nullptr;
   std::map<std::string, Tensor> inputs;              // the arrays parts asked for, on the GPU
@@ -126,6 +126,8 @@ class PositionEncoding : public Part {
   // elements c and c + half, the angle position * frequency) and the factor on every cosine and sine.
   virtual const Tensor* angle_frequencies() { return nullptr; }
   virtual float magnitude() { return 1.f; }
+  // true: pair c of such a rotation is a head's elements 2c and 2c + 1, not c and c + half.
+  virtual bool pairs_neighbours() const { return false; }
   // Encodes positions [T] into q [T, heads, d] and k [T, kv heads, d]; k may have no memory (only q is wanted).
   // The default rotates by the tables above; a kind without tables brings its own.
   virtual std::pair<Tensor, Tensor> apply(const Tensor& q, const Tensor& k, const Tensor& positions);

@@ -213,6 +213,7 @@ int vh_model_types(char* out, int cap) {
 }
 
 void vh_rotary_inverse_frequencies(double theta, int rotary_dim, float* out) { rotary_inverse_frequencies(theta, rotary_dim, out); }
+void vh_rotary_linear_frequencies(double theta, int rotary_dim, double factor, float* out) { rotary_linear_frequencies(theta, rotary_dim, factor, out); }
 float vh_rotary_stretched_frequencies(double theta, int rotary_dim, double factor, double original, double fast, double slow, float* out) {
   return rotary_stretched_frequencies(theta, rotary_dim, factor, original, fast, slow, out);
 }

@@ -9,6 +9,7 @@
 
 #include "qwen3.h"
 #include "pabavik.h"
+#include "pasovik.h"
 #include "povatar.h"
 #include "tezinex.h"
 
@@ -194,6 +195,7 @@ void register_builtin_architectures() {
   register_architecture("Tezinex", "tezinex", tezinex_model_spec);
   register_architecture("Povatar", "povatar", povatar_model_spec);
   register_architecture("Pabavik", "pabavik", pabavik_model_spec);
+  register_architecture("Pasovik", "pasovik", pasovik_model_spec);
 }
 
 }  // namespace vosti

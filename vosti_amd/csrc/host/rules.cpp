@@ -33,6 +33,10 @@ float rotary_stretched_frequencies(double theta, int rotary_dim, double factor, 
   return stretch ? (float)(0.1 * std::log(factor) + 1.0) : 1.0f;
 }
 
+void rotary_linear_frequencies(double theta, int rotary_dim, double factor, float* out) {
+  for (int j = 0; j < rotary_dim / 2; ++j) out[j] = (float)(std::pow(theta, -2.0 * j / rotary_dim) / factor);
+}
+
 static int bucket(int n) {      // the smallest of 1, 2, 3, 4, 6, 8, 12, 16, ... that is at least n
   for (int b = 1;; b *= 2) {
     if (b >= n) return b;

@@ -22,6 +22,10 @@ void rotary_inverse_frequencies(double theta, int rotary_dim, float* out);
 // factor <= 0: no stretch (out[j] = f[j], returns 1).
 float rotary_stretched_frequencies(double theta, int rotary_dim, double factor, double original, double fast, double slow, float* out);
 
+// The frequencies of a rotation whose positions are all stretched alike: out[j] = theta^(-2j / rotary_dim) / factor,
+// computed in 64-bit and rounded once.  factor 1: the plain frequencies.
+void rotary_linear_frequencies(double theta, int rotary_dim, double factor, float* out);
+
 // Recorded decode steps have one of 1, 2, 3, 4, 6, 8, 12, 16, 24, ... rows (a step with fewer is filled up with
 // rows that read one key and store nothing; the reference pads its graphs likewise,
 // python/vosti_kernels/graph_overlay.py:177-389), and block tables one of these numbers times eight pages, so

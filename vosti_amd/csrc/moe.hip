@@ -62,8 +62,10 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(float* __restrict__ z, 
 }
 
 // The choice: idx [T, top] int32, wts [T, top] floats from the logits.  One wave per token, four tokens a workgroup.
+// score 0: the softmax over all experts, the chosen scores divided by their sum plus weight_eps; score 1: the logistic
+// function of every logit, the chosen scores as they are (the order of the scores is the order of the logits either way).
 __global__ __launch_bounds__(256) void moe_choose_kernel(int32_t* __restrict__ idx, float* __restrict__ wts, const float* __restrict__ logits,
-                                                         int T, int E, int top, float weight_eps) {
+                                                         int T, int E, int top, float weight_eps, int score_kind) {
   extern __shared__ float scores[];      // [4][E]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int t = blockIdx.x * 4 + wave;
@@ -77,11 +79,11 @@ __global__ __launch_bounds__(256) void moe_choose_kernel(int32_t* __restrict__ i
   mx = wave_max_xor(mx);
   float sum = 0.f;
   for (int e = lane; e < E; e += 64) {
-    const float p = expf(z[e] - mx);
+    const float p = score_kind == 1 ? 1.f / (1.f + expf(-z[e])) : expf(z[e] - mx);
     z[e] = p;
     sum = sum + p;
   }
-  sum = wave_sum_xor(sum);
+  sum = score_kind == 1 ? 1.f : wave_sum_xor(sum);
   // The largest score `top` times; a chosen one is marked with -1 (scores are positive or zero).
   float chosen_sum = 0.f;
   float my_w = 0.f;
@@ -106,7 +108,7 @@ __global__ __launch_bounds__(256) void moe_choose_kernel(int32_t* __restrict__ i
     if (lane == 0) z[best_e] = -1.f;
     __builtin_amdgcn_wave_barrier();
   }
-  const float denom = chosen_sum + weight_eps;
+  const float denom = score_kind == 1 ? 1.f : chosen_sum + weight_eps;
   if (lane < top) {
     idx[(int64_t)t * top + lane] = my_e;
     wts[(int64_t)t * top + lane] = my_w / denom;
@@ -261,32 +263,47 @@ __global__ __launch_bounds__(256) void moe_relu_square_kernel(elem_t* x, int64_t
 // A gated expert's activation between its two products: row r of `in` holds the gate's F outputs and, from column F on,
 // the up projection's; y = g * sigmoid(slope * g) * (u + shift) with g = min(gate, limit) and u = clamp(up, -limit, limit),
 // in 32-bit, as elements [rows, F].  A thread takes a 16-byte vector (F in whole vectors).
+// row_pair / wts (both or neither): row r's gate and up values are multiplied by the weight of the row's (token, choice) pair
+// before they are clamped, which is what an expert computes that reads its input times that weight; a row without a pair
+// gives zeros.
 __global__ __launch_bounds__(256) void moe_glu_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ in, int64_t rows, int F, float limit,
-                                                      float slope, float shift) {
+                                                      float slope, float shift, const int32_t* __restrict__ row_pair, const float* __restrict__ wts) {
   const int per = F / VK_VEC;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= rows * per) return;
   const int64_t r = i / per;
   const int c = (int)(i - r * per) * VK_VEC;
   float g[VK_VEC], u[VK_VEC];
+  float rw = 1.f;
+  if (row_pair != nullptr) {
+    const int pair = row_pair[r];
+    if (pair < 0) {
+#pragma unroll
+      for (int j = 0; j < VK_VEC; ++j) g[j] = 0.f;
+      store_elems(out + r * F + c, g);
+      return;
+    }
+    rw = wts[pair];
+  }
   load_elems(in + r * 2 * F + c, g);
   load_elems(in + r * 2 * F + F + c, u);
 #pragma unroll
   for (int j = 0; j < VK_VEC; ++j) {
-    const float gc = fminf(g[j], limit), uc = fminf(fmaxf(u[j], -limit), limit);
+    const float gc = fminf(g[j] * rw, limit), uc = fminf(fmaxf(u[j] * rw, -limit), limit);
     g[j] = (gc / (1.f + expf(-slope * gc))) * (uc + shift);
   }
   store_elems(out + r * F + c, g);
 }
 
-// out[t, c] = sum over k < top, ascending, of wts[t, k] * y[pair_row[t * top + k], c], from zero; then + extra[t, c]
+// out[t, c] = sum over k < top, ascending, of wts[t, k] * y[pair_row[t * top + k], c] (wts null: every weight 1), from zero; then + extra[t, c]
 // (elements, the output of an expert that every token uses) where there is one.
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ out, const elem_t* __restrict__ y, const float* __restrict__ wts,
                                                           const int32_t* __restrict__ pair_row, int W, int top, const elem_t* __restrict__ extra) {
   const int t = blockIdx.x;
   for (int c = blockIdx.y * 256 + threadIdx.x; c < W; c += gridDim.y * 256) {
     float acc = 0.f;
-    for (int k = 0; k < top; ++k) acc = acc + wts[(int64_t)t * top + k] * to_f32(y[(int64_t)pair_row[(int64_t)t * top + k] * W + c]);
+    for (int k = 0; k < top; ++k)
+      acc = acc + (wts != nullptr ? wts[(int64_t)t * top + k] : 1.f) * to_f32(y[(int64_t)pair_row[(int64_t)t * top + k] * W + c]);
     if (extra != nullptr) acc = acc + to_f32(extra[(int64_t)t * W + c]);
     out[(int64_t)t * W + c] = acc;
   }
@@ -303,14 +320,14 @@ int vk_moe_max_tiles(int T, int top, int E, int tile_rows) {
 
 // logits: scratch [T, E] floats.  bias [E] (elements, or floats with bias_is_f32) or null.
 static int route_launch(int32_t* idx, float* wts, float* logits, const elem_t* h, const elem_t* router, const void* bias, int bias_is_f32, int T, int W,
-                        int E, int top, float weight_eps, hipStream_t st) {
+                        int E, int top, float weight_eps, hipStream_t st, int score_kind = 0) {
   VK_REQUIRE(T >= 0 && W > 0 && W % VK_VEC == 0 && E > 0 && top > 0 && top <= E && E <= 4096,
              "router: bad sizes T=%d W=%d E=%d top=%d (the width in whole 16-byte vectors, at most 4096 experts)", T, W, E, top);
   VK_REQUIRE(((uintptr_t)h % 16) == 0 && ((uintptr_t)router % 16) == 0, "router: operands must be 16-byte aligned");
   if (T == 0) return 0;
   moe_logits_kernel<<<dim3((T + MOE_ROUTE_TOKENS - 1) / MOE_ROUTE_TOKENS, E), 256, 0, st>>>(logits, h, router, T, W, E, bias, bias_is_f32);
   if (vk_check_launch("router (logits)")) return 1;
-  moe_choose_kernel<<<(T + 3) / 4, 256, (size_t)4 * E * sizeof(float), st>>>(idx, wts, logits, T, E, top, weight_eps);
+  moe_choose_kernel<<<(T + 3) / 4, 256, (size_t)4 * E * sizeof(float), st>>>(idx, wts, logits, T, E, top, weight_eps, score_kind);
   return vk_check_launch("router (choice)");
 }
 
@@ -325,6 +342,14 @@ int vk_moe_route_bias(int32_t* idx, float* wts, float* logits, const elem_t* h, 
                       int E, int top, float weight_eps, hipStream_t st) {
   VK_REQUIRE(bias != nullptr, "router: the bias is missing");
   return route_launch(idx, wts, logits, h, router, bias, bias_is_f32, T, W, E, top, weight_eps, st);
+}
+
+// The same with a choice of score: 0 is vk_moe_route (vk_moe_route_bias with a bias), 1 gives every chosen expert the
+// logistic function of its logit as its weight, not divided by anything.  bias may be null.
+int vk_moe_route_scored(int32_t* idx, float* wts, float* logits, const elem_t* h, const elem_t* router, const void* bias, int bias_is_f32, int T, int W,
+                        int E, int top, float weight_eps, int score_kind, hipStream_t st) {
+  VK_REQUIRE(score_kind == 0 || score_kind == 1, "router: score kind %d", score_kind);
+  return route_launch(idx, wts, logits, h, router, bias, bias_is_f32, T, W, E, top, weight_eps, st, score_kind);
 }
 
 int vk_moe_plan(const int32_t* idx, int32_t* row_pair, int32_t* row_token, int32_t* pair_row, int32_t* tile_expert, int32_t* expert_start, int T,
@@ -369,7 +394,20 @@ int vk_moe_glu(elem_t* out, const elem_t* in, int64_t rows, int F, float limit, 
              "experts (gated activation): bad sizes rows=%lld F=%d (whole 16-byte vectors)", (long long)rows, F);
   if (rows == 0) return 0;
   const int64_t n = rows * (F / VK_VEC);
-  moe_glu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(out, in, rows, F, limit, slope, shift);
+  moe_glu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(out, in, rows, F, limit, slope, shift, nullptr, nullptr);
+  return vk_check_launch("experts (gated activation)");
+}
+
+// The same for experts that read their input times the pair's weight: row r's gate and up values are multiplied by
+// wts[row_pair[r]] before the clamps (W (w h) = w (W h)); rows without a pair come out zero.
+int vk_moe_glu_weighed(elem_t* out, const elem_t* in, int64_t rows, int F, float limit, float slope, float shift, const int32_t* row_pair,
+                       const float* wts, hipStream_t st) {
+  VK_REQUIRE(rows >= 0 && F > 0 && F % VK_VEC == 0 && limit > 0.f && ((uintptr_t)out % 16) == 0 && ((uintptr_t)in % 16) == 0,
+             "experts (gated activation): bad sizes rows=%lld F=%d (whole 16-byte vectors)", (long long)rows, F);
+  VK_REQUIRE(row_pair != nullptr && wts != nullptr, "experts (gated activation): the rows' pairs and weights are missing");
+  if (rows == 0) return 0;
+  const int64_t n = rows * (F / VK_VEC);
+  moe_glu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(out, in, rows, F, limit, slope, shift, row_pair, wts);
   return vk_check_launch("experts (gated activation)");
 }
 

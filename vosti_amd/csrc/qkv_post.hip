@@ -32,6 +32,7 @@ struct QkvPostArgs {
   const int32_t* slots;      // [T]: page * P + offset, or -1
   int w_is_f32, nq, nkv, d, P, rot_half;
   int norm_d;             // the head norm's own size: the mean of squares divides by it, and its weight has this many entries
+  int neighbours;         // 1: pair c of a head is its elements 2c and 2c + 1 instead of c and c + rot_half
   float eps;
 };
 
@@ -57,7 +58,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a, int per_wa
   const int d = a.d, heads = a.nq + 2 * a.nkv;
   const int rh = a.rot_half;
   // With a rotation half of 64 or 128 elements the partner of an element is held by the same lane.
-  const bool in_lane = rh % 64 == 0;
+  const bool in_lane = rh % 64 == 0 && !a.neighbours;
   const int shift = rh / 64;
   const bool has_rot = a.cos_t != nullptr || a.inv_freq != nullptr;
   int64_t trow = 0;
@@ -107,7 +108,15 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a, int per_wa
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int c = lane + 64 * i;
-        if (c < rh) {
+        if (a.neighbours) {
+          // Element 2c is the pair's first, 2c + 1 its second; both lie in y.
+          if (c < 2 * rh) {
+            float cs, sn;
+            pair_angle(a, trow, posf, c >> 1, cs, sn);
+            const float other = y[c ^ 1];
+            xv[i] = (c & 1) ? old[i] * cs + other * sn : old[i] * cs - other * sn;
+          }
+        } else if (c < rh) {
           float cs, sn;
           pair_angle(a, trow, posf, c, cs, sn);
           const float other = in_lane ? (i + shift < 4 ? old[(i + shift) & 3] : 0.f) : y[c + rh];
@@ -241,7 +250,8 @@ extern "C" {
 static int qkv_post_launch(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc, elem_t* vc, const void* q_w,
                            const void* k_w, int w_is_f32, const elem_t* cos_t, const elem_t* sin_t, int rot_half,
                            const int32_t* positions, const int32_t* slots, int T, int nq, int nkv, int d, int P, float eps,
-                           const elem_t* bias, hipStream_t st, const float* inv_freq = nullptr, float mag = 1.f, int norm_d = 0) {
+                           const elem_t* bias, hipStream_t st, const float* inv_freq = nullptr, float mag = 1.f, int norm_d = 0,
+                           int neighbours = 0) {
   VK_REQUIRE(T >= 0 && nq >= 0 && nkv >= 0 && nq + nkv > 0, "qkv_post: bad sizes T=%d nq=%d nkv=%d", T, nq, nkv);
   VK_REQUIRE(d > 0 && d <= 256, "qkv_post: head size %d must be in 1..256", d);
   VK_REQUIRE(row_stride >= (int64_t)(nq + 2 * nkv) * d, "qkv_post: row stride %lld too small", (long long)row_stride);
@@ -259,6 +269,8 @@ static int qkv_post_launch(const elem_t* qkv, int64_t row_stride, elem_t* q_out,
   a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.slots = slots; a.w_is_f32 = w_is_f32; a.bias = bias;
   a.nq = nq; a.nkv = nkv; a.d = d; a.P = P; a.rot_half = rot_half; a.eps = eps; a.inv_freq = inv_freq; a.mag = mag;
   a.norm_d = norm_d;
+  a.neighbours = neighbours;
+  VK_REQUIRE(!neighbours || inv_freq != nullptr, "qkv_post: neighbouring pairs are built for computed angles");
   // Few tokens: four waves' worth of heads per workgroup, for many workgroups; many tokens: all heads of a token.
   const int heads = nq + 2 * nkv;
   const int lph = d / VK_VEC;          // lanes per head in the kernel with 16-byte accesses
@@ -317,6 +329,20 @@ int vk_qkv_post_norm_angles(const elem_t* qkv, int64_t row_stride, elem_t* q_out
   VK_REQUIRE(norm_d > 0 && 2 * rot_half <= norm_d, "qkv_post: a rotation of %d elements in a head norm of %d", 2 * rot_half, norm_d);
   return qkv_post_launch(qkv, row_stride, q_out, kc, vc, q_w, k_w, w_is_f32, nullptr, nullptr, rot_half, positions, slots, T, nq, nkv, d, P, eps,
                          nullptr, st, inv_freq, mag, norm_d);
+}
+
+// The same with a choice of which elements form a pair: neighbours 1 turns the elements 2c and 2c + 1 of a head by
+// position * inv_freq[c] (c < rot_half), 0 is vk_qkv_post_norm_angles.  q_w and k_w may both be null (no head norms; norm_d
+// is then not used).
+int vk_qkv_post_norm_angles_paired(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc, elem_t* vc, const void* q_w, const void* k_w,
+                                   int w_is_f32, int norm_d, float eps, const float* inv_freq, float mag, int rot_half, int neighbours,
+                                   const int32_t* positions, const int32_t* slots, int T, int nq, int nkv, int d, int P, hipStream_t st) {
+  VK_REQUIRE(inv_freq != nullptr, "qkv_post: the rotation's frequencies are missing");
+  VK_REQUIRE(neighbours == 0 || neighbours == 1, "qkv_post: 'neighbours' is 0 or 1");
+  const bool normed = q_w != nullptr || k_w != nullptr;
+  VK_REQUIRE(!normed || (norm_d > 0 && 2 * rot_half <= norm_d), "qkv_post: a rotation of %d elements in a head norm of %d", 2 * rot_half, norm_d);
+  return qkv_post_launch(qkv, row_stride, q_out, kc, vc, q_w, k_w, w_is_f32, nullptr, nullptr, rot_half, positions, slots, T, nq, nkv, d, P, eps,
+                         nullptr, st, inv_freq, mag, normed ? norm_d : 0, neighbours);
 }
 
 }  // extern "C"

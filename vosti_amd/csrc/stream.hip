@@ -285,6 +285,24 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_pair_norm_vec_kernel(fl
   }
 }
 
+// out[t, c] = gelu(gate[t, c]) * table[ids[t], first + c] for c < n, zero for n <= c < ldo: a token's slice of a second
+// embedding table, gated by a projection of the stream.  gelu(z) = z / 2 * (1 + tanh(sqrt(2 / pi) * (z + 0.044715 z^3))), in 32-bit.
+__global__ __launch_bounds__(256) void side_gate_kernel(elem_t* __restrict__ out, int64_t ldo, const elem_t* __restrict__ gate, int64_t ldg,
+                                                        const elem_t* __restrict__ table, int64_t table_width, const int32_t* __restrict__ ids, int first,
+                                                        int n, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / ldo;
+  const int c = (int)(i - t * ldo);
+  float v = 0.f;
+  if (c < n) {
+    const float z = to_f32(gate[t * ldg + c]);
+    const float inner = 0.7978845608028654f * (z + 0.044715f * ((z * z) * z));
+    v = ((0.5f * z) * (1.f + tanhf(inner))) * to_f32(table[(int64_t)ids[t] * table_width + first + c]);
+  }
+  out[i] = from_f32<elem_t>(v);
+}
+
 extern "C" {
 
 int vk_embed_sinusoid(float* out, const elem_t* table, const int32_t* ids, const int32_t* positions, const float* inv_freq, int T,
@@ -396,6 +414,17 @@ int vk_stream_pair_norm(float* out, const elem_t* a, const void* wa, const elem_
     stream_pair_norm_kernel<<<rows, STREAM_THREADS, 0, st>>>(out, a, wa, b, wb, w_is_f32, H, eps, ca, cb);
   }
   return vk_check_launch("pair norm");
+}
+
+// out [T, ldo] elements from gate [T, ldg] (its first n columns) and the columns [first, first + n) of table [V, table_width]
+// at the rows ids name; the columns of out beyond n are zero.  Ids must lie below V: the caller checks them on the host.
+int vk_side_gate(elem_t* out, int64_t ldo, const elem_t* gate, int64_t ldg, const elem_t* table, int64_t table_width, const int32_t* ids, int first,
+                 int n, int T, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && n > 0 && first >= 0 && ldo >= n && ldg >= n && table_width >= (int64_t)first + n, "token side input: bad sizes n=%d first=%d", n, first);
+  if (T == 0) return 0;
+  const int64_t total = (int64_t)T * ldo;
+  side_gate_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(out, ldo, gate, ldg, table, table_width, ids, first, n, total);
+  return vk_check_launch("token side input");
 }
 
 }  // extern "C"

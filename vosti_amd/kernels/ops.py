@@ -15,7 +15,7 @@ import torch
 
 from . import build
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 SEGMENT_KEYS = 256
 ATTN_ITEM_ROWS = 128      # rows of one prompt item of paged_attention
 
