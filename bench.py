@@ -6,6 +6,7 @@
     python bench.py --workload mixed14b     # Qwen3-14B shape: 32 prompts of 128 to 4,096 tokens, prefill in portions beside decoding
     python bench.py --workload prefix32b    # Qwen3-32B shape: 64 requests at context 8,192 that share a 1,024-token prefix
     python bench.py --workload aligned      # the reference's aligned phases: batch 4, cached contexts 0 to 16K, 256 new tokens / 127 decode steps
+    python bench.py --workload pasovik      # the Pasovik design (attention through a latent, linear attention with fixed decays, a second embedding a layer) at three layer sizes beside Pabavik at equal size
     python bench.py --workload pabavik      # the Pabavik design (gated linear attention, windowed attention with an output gate, gated experts beside a shared one) at three layer sizes beside Tezinex at equal size
     python bench.py --workload povatar      # the Povatar design (attention beside a state-space recurrence, routed experts) at three layer sizes beside Tezinex at equal size
     python bench.py --workload tezinex      # the Tezinex design at three layer sizes beside the Qwen3 decoder at equal size: prefill and decode
@@ -88,9 +89,9 @@ def main() -> int:
     ap.add_argument("--no-other-shapes", action="store_true", help="skip the 14B and 32B workloads that the default record holds as points")
     ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
                     help="context length of the decode measurement (the prefill figure is always of 2,048 tokens)")
-    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b", "aligned", "tezinex", "povatar", "pabavik"])
-    ap.add_argument("--sizes", default=",".join(["1k", "2k", "4k"]), help="which layer sizes --workload tezinex / povatar / pabavik measure (1k, 2k, 4k)")
-    ap.add_argument("--only-design", default="", choices=["", "tezinex", "qwen3", "povatar", "pabavik"], help="--workload tezinex / povatar / pabavik: measure one of the two designs only")
+    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b", "aligned", "tezinex", "povatar", "pabavik", "pasovik"])
+    ap.add_argument("--sizes", default=",".join(["1k", "2k", "4k"]), help="which layer sizes --workload tezinex / povatar / pabavik / pasovik measure (1k, 2k, 4k)")
+    ap.add_argument("--only-design", default="", choices=["", "tezinex", "qwen3", "povatar", "pabavik", "pasovik"], help="--workload tezinex / povatar / pabavik / pasovik: measure one of the two designs only")
     ap.add_argument("--engine", default="native", choices=["native", "python"],
                     help="which engine every figure is measured through: the native one (vosti_amd.engine.NativeEngine) or the "
                          "Python step function over the same kernels, cache manager and scheduler")
@@ -113,7 +114,7 @@ def main() -> int:
     if args.workload == "aligned":
         print(json.dumps(aligned_workload(args)), flush=True)
         return 0
-    if args.workload in ("tezinex", "povatar", "pabavik"):
+    if args.workload in ("tezinex", "povatar", "pabavik", "pasovik"):
         print(json.dumps(tezinex_workload(args)), flush=True)
         return 0
     if args.workload != "decode8b":
@@ -567,11 +568,41 @@ def pabavik_config(width, heads, kv_heads, ff, layers, vocab):
             "width": width}
 
 
+def pasovik_config(width, heads, kv_heads, ff, layers, vocab):
+    """Linear attention with a fixed decay a head, attention, attention through a latent, attention on the latent of the one
+    before, ... (heads of 128 and a state of Pabavik's size; a latent of 192 beside 64 rotated entries, which fills the
+    attention kernels' widest head), a dense feed-forward under the first and third and 32 experts a quarter as wide, of which
+    a token uses 4, under the others, and a second embedding of 256 columns a layer: a token's matrix work is about that of a
+    Pabavik or Tezinex layer of these sizes."""
+    dense = {"kind": "dense", "ff": ff}
+    experts = {"kind": "moe", "expert": {"ff": ff // 4, "limit": 7.0}, "router": {"experts": 32, "top": 4}}
+    decay = [1.0 - 2.0 ** (-5.0 - 5.0 * h / max(heads - 1, 1)) for h in range(heads)]
+
+    def latent(kv_from=None):
+        m = {"dim": 128, "rot_dim": 64, "vdim": 128, "heads": heads, "kv_rank": 192, "q_rank": width // 2, "scale": 192 ** -0.5,
+             "rot": {"base": 10000.0, "dims": 64}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return m
+    out = []
+    for i in range(layers):
+        kind = i % 4
+        if kind == 0:
+            out.append({"type": "lightning", "mixer": {"dim": 128, "vdim": 128, "heads": heads, "decay": decay}, "mlp": dense})
+        elif kind == 1:
+            out.append({"type": "attention", "mlp": experts,
+                        "mixer": {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": kv_heads, "scale": 128 ** -0.5, "softcap": 20.0,
+                                  "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0}}}})
+        else:
+            out.append({"type": "latent_attention", "mixer": latent(i - 1 if kind == 3 else None), "mlp": dense if kind == 2 else experts})
+    return {"architecture": "Pasovik", "layers": out, "norm": {"eps": 1e-5}, "token_side": {"dim": 256}, "vocab": vocab, "width": width}
+
+
 def tezinex_workload(args) -> dict:
     """Prefill of one prompt and decoding at a fixed batch for the Tezinex design at three layer sizes, each beside the
     Qwen3 decoder with the same width, heads, feed-forward, layers and vocabulary (random weights, the native engine).
     --workload povatar: the Povatar design beside Tezinex, its nearest neighbour here, in the same way; --workload pabavik:
-    the Pabavik design beside Tezinex."""
+    the Pabavik design beside Tezinex; --workload pasovik: the Pasovik design beside Pabavik."""
     import tempfile
     from vosti_amd.engine import NativeEngine
     from vosti_amd.sampling import SamplingParams
@@ -583,7 +614,8 @@ def tezinex_workload(args) -> dict:
     record = {"metric": "decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
               "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
               "data": "synthetic: seeded random token prompts, seeded random weights", "sizes": {},
-              "config": {"model": "Pabavik (linear attention, attention, shared-key attention, linear attention, ...; 32 experts of which 3 and a shared one) beside Tezinex at equal size"
+              "config": {"model": "Pasovik (linear attention, attention, latent attention, attention on the latent before, ...; dense layers and 32 experts of which 4; a second embedding) beside Pabavik at equal size"
+                         if args.workload == "pasovik" else "Pabavik (linear attention, attention, shared-key attention, linear attention, ...; 32 experts of which 3 and a shared one) beside Tezinex at equal size"
                          if args.workload == "pabavik" else "Povatar (attention beside a state-space recurrence, 32 experts of which 4) beside Tezinex at equal size"
                          if args.workload == "povatar" else "Tezinex (delta, attention, shared-key attention, delta, ...) beside Qwen3 at equal size",
                          "layers": layers,
@@ -630,12 +662,16 @@ def tezinex_workload(args) -> dict:
 
     # The design that is measured and the neighbour it stands beside.
     first, second = (args.workload, "tezinex") if args.workload in ("povatar", "pabavik") else ("tezinex", "qwen3")
+    if args.workload == "pasovik":
+        first, second = "pasovik", "pabavik"
 
     def config_of(design, width, heads, kv_heads, ff):
         if design == "povatar":
             return povatar_config(width, heads, kv_heads, ff, layers, vocab)
         if design == "pabavik":
             return pabavik_config(width, heads, kv_heads, ff, layers, vocab)
+        if design == "pasovik":
+            return pasovik_config(width, heads, kv_heads, ff, layers, vocab)
         if design == "tezinex":
             return tezinex_config(width, heads, kv_heads, ff, layers, vocab)
         return dict(QWEN3_8B, architectures=["Qwen3ForCausalLM"], vocab_size=vocab, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,

@@ -128,7 +128,7 @@ def test_usage_errors(program, tmp_path):
     r = subprocess.run([program, "--family", "qwen3"], capture_output=True, text=True, env={})
     assert r.returncode == 2 and "MODEL_PATH (or --model-path) is required" in r.stderr
     r = subprocess.run([program, "--family", "llama", "--model-path", str(tmp_path)], capture_output=True, text=True, env={})
-    assert r.returncode == 2 and "unknown --family llama (one of: pabavik, povatar, qwen3, tezinex)" in r.stderr
+    assert r.returncode == 2 and "unknown --family llama (one of: pabavik, pasovik, povatar, qwen3, tezinex)" in r.stderr
     r = subprocess.run([program, "--family", "qwen3", "--model-path", str(tmp_path), "--colour", "blue"], capture_output=True, text=True, env={})
     assert r.returncode == 2 and "unknown option --colour" in r.stderr
 

@@ -98,7 +98,7 @@ def test_without_the_plugin_the_architecture_is_unknown(toy_dirs, tmp_path):
     args = [program, "--family", "toy_scaled_rope", "--dtype", "float32", "--lib-dir", str(lib.parent), "--model-path", str(toy_dirs["B"]),
             "--prompt-ids", "5,17,3,99", "--max-tokens", "6", "--page-size", "8"]
     r = subprocess.run(args, capture_output=True, text=True, timeout=110, env={})
-    assert r.returncode == 2 and "unknown --family toy_scaled_rope (one of: pabavik, povatar, qwen3, tezinex)" in r.stderr
+    assert r.returncode == 2 and "unknown --family toy_scaled_rope (one of: pabavik, pasovik, povatar, qwen3, tezinex)" in r.stderr
     so = build.build_plugin(ROOT / "tests" / "toy_plugin.cpp", tmp_path / "toy_plugin.so")
     r = subprocess.run(args + ["--plugin", str(so)], capture_output=True, text=True, timeout=110, env={})
     assert r.returncode == 0, r.stderr[-2000:]

@@ -115,6 +115,18 @@ def rotary_inverse_frequencies(theta: float, rotary_dim: int):
     return out
 
 
+def rotary_linear_frequencies(theta: float, rotary_dim: int, factor: float = 1.0):
+    """float32 numpy array [rotary_dim / 2]: theta^(-2j / rotary_dim) / factor, as the engine's rotary_stretched part computes
+    them for a ``linear_factor``."""
+    import numpy as np
+    out = np.empty(rotary_dim // 2, dtype=np.float32)
+    lib = host_lib()
+    lib.vh_rotary_linear_frequencies.restype = None
+    lib.vh_rotary_linear_frequencies.argtypes = [ctypes.c_double, ctypes.c_int, ctypes.c_double, ctypes.c_void_p]
+    lib.vh_rotary_linear_frequencies(float(theta), int(rotary_dim), float(factor), out.ctypes.data)
+    return out
+
+
 def rotary_stretched_frequencies(theta: float, rotary_dim: int, factor: float = 0.0, original: float = 1.0, fast: float = 1.0, slow: float = 1.0):
     """(float32 numpy array [rotary_dim / 2], factor on cosine and sine): the frequencies of a rotation whose long
     wavelengths are stretched by ``factor`` (0: not at all), as the engine's rotary_stretched part computes them."""

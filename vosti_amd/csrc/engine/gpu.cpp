@@ -141,6 +141,8 @@ struct Kernels::Fn {
   int (*moe_combine_add)(P, CP, CP, CP, CP, int, int, int, hipStream_t);
   int (*stream_norm_add_f32)(P, CP, CP, CP, int, int, int, float, float, float, hipStream_t);
   int (*cast_from_f32)(P, CP, int64_t, hipStream_t);
+  int (*stream_norm_add_rounded)(P, CP, CP, CP, int, int, int, float, float, float, P, hipStream_t);
+  int (*stream_norm_add_f32_rounded)(P, CP, CP, CP, int, int, int, float, float, float, P, hipStream_t);
   int (*moe_route_scored)(P, P, P, CP, CP, CP, int, int, int, int, int, float, int, hipStream_t);
   int (*moe_glu_weighed)(P, CP, int64_t, int, float, float, float, CP, CP, hipStream_t);
   int (*norm_columns)(P, int64_t, CP, int64_t, int, int, CP, int, float, int, hipStream_t);
@@ -189,6 +191,7 @@ Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(na
   VK(qkv_post_norm_angles, "vk_qkv_post_norm_angles"); VK(gate_mul, "vk_gate_mul"); VK(gla_decay, "vk_gla_decay"); VK(gla_rule, "vk_gla_rule");
   VK(gated_head_norm, "vk_gated_head_norm"); VK(moe_route_bias, "vk_moe_route_bias"); VK(moe_up_plain, "vk_moe_up_plain"); VK(moe_glu, "vk_moe_glu");
   VK(moe_combine_add, "vk_moe_combine_add"); VK(stream_norm_add_f32, "vk_stream_norm_add_f32");
+  VK(stream_norm_add_rounded, "vk_stream_norm_add_rounded"); VK(stream_norm_add_f32_rounded, "vk_stream_norm_add_f32_rounded");
   VK(cast_from_f32, "vk_cast_from_f32"); VK(moe_route_scored, "vk_moe_route_scored"); VK(moe_glu_weighed, "vk_moe_glu_weighed");
   VK(norm_columns, "vk_norm_columns"); VK(gemm_heads, "vk_gemm_heads"); VK(latent_post, "vk_latent_post");
   VK(qkv_post_norm_angles_paired, "vk_qkv_post_norm_angles_paired"); VK(linear_rule, "vk_linear_rule"); VK(side_gate, "vk_side_gate");
@@ -481,12 +484,18 @@ Tensor Kernels::stream_norm(const Tensor& x, const Tensor& w, float eps, float o
   return out;
 }
 
-void Kernels::stream_norm_add(Tensor& out, const Tensor& base, const Tensor& y, const Tensor& w, float eps, float offset, float mult) {
+void Kernels::stream_norm_add(Tensor& out, const Tensor& base, const Tensor& y, const Tensor& w, float eps, float offset, float mult, Tensor* rounded) {
   if (y.dtype != DType::F32) expect(y, "norm input", dtype_);
   if (y.shape.size() != 2) throw EngineError("norm input is " + y.describe());
   expect(base, "stream", DType::F32, y.shape);
   expect(out, "stream", DType::F32, y.shape);
   const int wf = norm_weight(w, "norm weight", y.dim(1));
+  if (rounded) {
+    expect(*rounded, "the stream's rounded rows", dtype_, y.shape);
+    auto fn = (y.dtype == DType::F32 && dtype_ != DType::F32) ? fn_->stream_norm_add_f32_rounded : fn_->stream_norm_add_rounded;
+    call(fn(out.data, base.data, y.data, w.data, wf, (int)y.dim(0), (int)y.dim(1), eps, offset, mult, rounded->data, stream));
+    return;
+  }
   // A sublayer's rows may be elements or, where it left them unrounded, floats.
   if (y.dtype == DType::F32 && dtype_ != DType::F32) {
     call(fn_->stream_norm_add_f32(out.data, base.data, y.data, w.data, wf, (int)y.dim(0), (int)y.dim(1), eps, offset, mult, stream));

@@ -143,7 +143,8 @@ class Kernels {
   // x (floats or elements) * rsqrt(mean(x^2) + eps) * (offset + w), as elements.
   Tensor stream_norm(const Tensor& x, const Tensor& w, float eps, float offset);
   // out = base + mult * norm(y), floats; out may be base.
-  void stream_norm_add(Tensor& out, const Tensor& base, const Tensor& y, const Tensor& w, float eps, float offset, float mult);
+  // rounded (elements of out's shape, or null): the new rows rounded to elements as well.
+  void stream_norm_add(Tensor& out, const Tensor& base, const Tensor& y, const Tensor& w, float eps, float offset, float mult, Tensor* rounded = nullptr);
   // out = sum over j < n of coef[j] * states[j]; states [>= n, ...] floats.
   Tensor stream_mix(const Tensor& states, const Tensor& coef, int n);
   void softcap(Tensor& x, float cap);          // x <- cap * tanh(x / cap)

@@ -92,8 +92,8 @@ std::pair<Tensor, Tensor> PositionEncoding::apply(const Tensor& q, const Tensor&
   return {rotate(q), k.data ? rotate(k) : Tensor()};
 }
 
-void Norm::forward_scaled_add(const Tensor& y, const Tensor& base, Tensor& out, float mult) {
-  (void)y; (void)base; (void)out; (void)mult;
+void Norm::forward_scaled_add(const Tensor& y, const Tensor& base, Tensor& out, float mult, Tensor* rounded) {
+  (void)y; (void)base; (void)out; (void)mult; (void)rounded;
   throw EngineError("this norm kind cannot add its scaled output to a 32-bit residual stream");
 }
 
@@ -268,8 +268,8 @@ class RMSNorm : public Norm {
     if (offset_ != 0.f) throw EngineError("a norm with a weight offset has no fused residual add in the element type");
     return kernels.add_rmsnorm(x, residual, weight_, eps_);
   }
-  void forward_scaled_add(const Tensor& y, const Tensor& base, Tensor& out, float mult) override {
-    kernels.stream_norm_add(out, base, y, weight_, eps_, offset_, mult);
+  void forward_scaled_add(const Tensor& y, const Tensor& base, Tensor& out, float mult, Tensor* rounded) override {
+    kernels.stream_norm_add(out, base, y, weight_, eps_, offset_, mult, rounded);
   }
   const Tensor* row_scale_weight() const override { return offset_ == 0.f ? &weight_ : nullptr; }
   float eps() const override { return eps_; }
@@ -1569,9 +1569,30 @@ class PostNormBlock : public Block {
     if (hidden.dtype != DType::F32 || hidden.shape.size() != 2 || hidden.dim(1) != hidden_)
       throw EngineError("a post_norm block takes the 32-bit residual stream, not " + hidden.describe());
     Tensor stream = hidden;
-    norms_["mixer_out"]->forward_scaled_add(mixer_->forward(k.to_elements(stream), ctx, cache), stream, stream, 1.f);
-    if (has_ffn_) norms_["ffn_out"]->forward_scaled_add(ffn_->forward(k.to_elements(stream), ctx), stream, stream, 1.f);
-    if (side_) norms_["side_out"]->forward_scaled_add(side_->forward(k.to_elements(stream), ctx), stream, stream, 1.f);
+    // What the next sublayer reads, the stream rounded to elements, is written by the launch that adds to the stream; the
+    // layer's first sublayer finds what the layer before left (ctx.carry), or rounds the stream itself.  Where the elements
+    // are 32-bit the stream is read as it is.
+    const bool narrow = k.dtype() != DType::F32;
+    Tensor read;
+    auto left = ctx.carry.find("stream.rounded");
+    if (!narrow) read = stream;
+    else if (left != ctx.carry.end() && ctx.carry["stream.rounded_of"].data == stream.data && left->second.shape == stream.shape) read = left->second;
+    else read = k.to_elements(stream);
+    auto add = [&](const char* norm, const Tensor& y) {
+      if (!narrow) {
+        norms_[norm]->forward_scaled_add(y, stream, stream, 1.f);
+        return;
+      }
+      read = k.empty(stream.shape);
+      norms_[norm]->forward_scaled_add(y, stream, stream, 1.f, &read);
+    };
+    add("mixer_out", mixer_->forward(read, ctx, cache));
+    if (has_ffn_) add("ffn_out", ffn_->forward(read, ctx));
+    if (side_) add("side_out", side_->forward(read, ctx));
+    if (narrow) {
+      ctx.carry["stream.rounded"] = read;
+      ctx.carry["stream.rounded_of"] = stream;
+    }
     return {stream, residual};
   }
 

@@ -112,8 +112,9 @@ class Norm : public Part {
   // A norm that is y = x * rsqrt(mean(x^2) + eps) * w says so; a mixer may then run it inside a launch of its own.
   virtual const Tensor* row_scale_weight() const { return nullptr; }
   virtual float eps() const { return 0.f; }
-  // out = base + mult * norm(y) on a residual stream that is kept in 32-bit; out may be base.
-  virtual void forward_scaled_add(const Tensor& y, const Tensor& base, Tensor& out, float mult);
+  // out = base + mult * norm(y) on a residual stream that is kept in 32-bit; out may be base.  rounded (or null): elements of
+  // out's shape that receive the new rows rounded, for a sublayer that reads the stream as it is.
+  virtual void forward_scaled_add(const Tensor& y, const Tensor& base, Tensor& out, float mult, Tensor* rounded = nullptr);
 };
 
 class PositionEncoding : public Part {

@@ -67,7 +67,7 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_norm_kernel(elem_t* __r
 template <typename Y>     // the normed rows: elements, or floats
 __global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_kernel(float* out, const float* base_rows, const Y* __restrict__ y,
                                                                          const void* __restrict__ w, int w_is_f32, int H, float eps,
-                                                                         float offset, float mult) {
+                                                                         float offset, float mult, elem_t* __restrict__ rounded) {
   __shared__ float red[4];
   const int64_t base = (int64_t)blockIdx.x * H;
   float part = 0.f;
@@ -79,7 +79,9 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_kernel(float* 
   for (int c = threadIdx.x; c < H; c += STREAM_THREADS) {
     const float v = to_f32(y[base + c]);
     const float n = (v * rr) * (offset + load_weight(w, w_is_f32, c));
-    out[base + c] = base_rows[base + c] + mult * n;
+    const float o = base_rows[base + c] + mult * n;
+    out[base + c] = o;
+    if (rounded != nullptr) rounded[base + c] = from_f32<elem_t>(o);      // the new stream as the next sublayer reads it
   }
 }
 
@@ -128,7 +130,7 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_norm_vec_kernel(elem_t*
 template <int NV, typename Y>
 __global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_vec_kernel(float* out, const float* base_rows, const Y* __restrict__ y,
                                                                              const void* __restrict__ w, int w_is_f32, int H, float eps,
-                                                                             float offset, float mult) {
+                                                                             float offset, float mult, elem_t* __restrict__ rounded) {
   __shared__ float red[4];
   const int64_t base = (int64_t)blockIdx.x * H;
   const int nvec = H / 4;
@@ -159,6 +161,10 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_vec_kernel(flo
       o.z = b[j].z + mult * ((v[j].z * rr) * (offset + load_weight(w, w_is_f32, 4 * c + 2)));
       o.w = b[j].w + mult * ((v[j].w * rr) * (offset + load_weight(w, w_is_f32, 4 * c + 3)));
       *reinterpret_cast<f32x4*>(out + base + 4 * c) = o;
+      if (rounded != nullptr) {
+        elem_t* r = rounded + base + 4 * c;
+        r[0] = from_f32<elem_t>(o.x); r[1] = from_f32<elem_t>(o.y); r[2] = from_f32<elem_t>(o.z); r[3] = from_f32<elem_t>(o.w);
+      }
     }
   }
 }
@@ -335,16 +341,16 @@ int vk_stream_norm(elem_t* out, const void* x, int x_is_f32, const void* w, int 
 extern "C++" {
 template <typename Y>
 static int norm_add_launch(float* out, const float* base, const Y* y, const void* w, int w_is_f32, int rows, int H, float eps, float offset, float mult,
-                           hipStream_t st) {
+                           hipStream_t st, elem_t* rounded = nullptr) {
   VK_REQUIRE(rows >= 0 && H > 0 && eps >= 0.f, "stream norm-add: bad sizes rows=%d H=%d", rows, H);
   if (rows == 0) return 0;
   const int nv = (H / 4 + STREAM_THREADS - 1) / STREAM_THREADS;
   if (H % 4 == 0 && nv <= 8 && (uintptr_t)out % 16 == 0 && (uintptr_t)base % 16 == 0) {
-#define NORM_ADD_VEC(NV) stream_norm_add_vec_kernel<NV, Y><<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult)
+#define NORM_ADD_VEC(NV) stream_norm_add_vec_kernel<NV, Y><<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult, rounded)
     if (nv <= 1) NORM_ADD_VEC(1); else if (nv <= 2) NORM_ADD_VEC(2); else if (nv <= 4) NORM_ADD_VEC(4); else NORM_ADD_VEC(8);
 #undef NORM_ADD_VEC
   } else {
-    stream_norm_add_kernel<Y><<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult);
+    stream_norm_add_kernel<Y><<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult, rounded);
   }
   return vk_check_launch("stream norm-add");
 }
@@ -359,6 +365,19 @@ int vk_stream_norm_add(float* out, const float* base, const elem_t* y, const voi
 int vk_stream_norm_add_f32(float* out, const float* base, const float* y, const void* w, int w_is_f32, int rows, int H, float eps,
                            float offset, float mult, hipStream_t st) {
   return norm_add_launch<float>(out, base, y, w, w_is_f32, rows, H, eps, offset, mult, st);
+}
+
+// The same two, and the new rows of the stream rounded to elements as well (rounded [rows, H]): what a sublayer that reads
+// the stream as it is takes next, without a launch of its own.
+int vk_stream_norm_add_rounded(float* out, const float* base, const elem_t* y, const void* w, int w_is_f32, int rows, int H, float eps, float offset,
+                               float mult, elem_t* rounded, hipStream_t st) {
+  VK_REQUIRE(rounded != nullptr, "stream norm-add: the rounded rows have no memory");
+  return norm_add_launch<elem_t>(out, base, y, w, w_is_f32, rows, H, eps, offset, mult, st, rounded);
+}
+int vk_stream_norm_add_f32_rounded(float* out, const float* base, const float* y, const void* w, int w_is_f32, int rows, int H, float eps, float offset,
+                                   float mult, elem_t* rounded, hipStream_t st) {
+  VK_REQUIRE(rounded != nullptr, "stream norm-add: the rounded rows have no memory");
+  return norm_add_launch<float>(out, base, y, w, w_is_f32, rows, H, eps, offset, mult, st, rounded);
 }
 
 int vk_stream_mix(float* out, const float* states, int64_t stride, const void* coef, int coef_is_f32, int n, int64_t numel,
