@@ -153,15 +153,14 @@ struct RuleShape {
 
 //
 // DELTA false is the same walk without the correction: S <- diag(g) S + k v^T; o = S^T q (gated linear attention); beta is
-// not read, q is multiplied by q_scale as it is brought in, and the inputs may be elements (IN).  head_decay: one decay a
-// head [H] that takes the place of the decays per token and channel; in_act 1: q, k and v pass silu as they are brought in.
-template <int R, int DR, bool DELTA, typename IN>
+// not read, q is multiplied by q_scale as it is brought in, and the inputs may be elements (IN).  HEAD_DECAY: `decay` holds
+// one decay a head [H] that takes the place of the decays per token and channel.
+template <int R, int DR, bool DELTA, typename IN, bool HEAD_DECAY = false>
 __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restrict__ out, const IN* __restrict__ qkv, int64_t ld, int q_col,
                                                                   int k_col, int v_col, const float* __restrict__ decay,
                                                                   const elem_t* __restrict__ b, int64_t ldb, float* state, int64_t state_stride,
                                                                   const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
-                                                                  const int32_t* __restrict__ slots, int H, int G, int d, int dv, float q_scale,
-                                                                  const float* __restrict__ head_decay, int in_act) {
+                                                                  const int32_t* __restrict__ slots, int H, int G, int d, int dv, float q_scale) {
   using Sh = RuleShape<R, DR>;
   constexpr int DMAX = Sh::DMAX, TC = Sh::TC, CB = Sh::CB;
   __shared__ __attribute__((aligned(16))) float smem[2 * Sh::BUF];
@@ -198,6 +197,7 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
   // What this thread brings in of a chunk: elements e = tid, tid + 256, ... of the chunk's [TC][DMAX] tiles of k, q and
   // the decays, and of its [TC][CB] tile of v; beta by the first TC threads.  Channels beyond d read as k = q = 0, g = 1.
   float pk[Sh::NI], pq[Sh::NI], pg[Sh::NI], pv[Sh::NV], pb = 0.f;
+  const float head_g = HEAD_DECAY ? decay[h] : 1.f;
   auto fetch = [&](int chunk) {
     const int t0 = chunk * TC;
 #pragma unroll
@@ -207,13 +207,9 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
       const bool ok = e < TC * DMAX && t0 + tok < n && c < d;
       const int64_t t = first + t0 + (ok ? tok : 0);
       const int cc = ok ? c : 0;
-      float kv = to_f32(qkv[t * ld + k_col + (int64_t)g * d + cc]), qv = to_f32(qkv[t * ld + q_col + (int64_t)g * d + cc]);
-      if (in_act) {
-        kv = silu_f(kv);
-        qv = silu_f(qv);
-      }
-      // One decay a head for all tokens and channels, or one per token and channel.
-      const float gv = head_decay != nullptr ? head_decay[h] : decay[(t * H + h) * d + cc];
+      const float kv = to_f32(qkv[t * ld + k_col + (int64_t)g * d + cc]), qv = to_f32(qkv[t * ld + q_col + (int64_t)g * d + cc]);
+      // One decay a head for all tokens and channels (decay [H]), or one per token and channel (decay [T, H, d]).
+      const float gv = HEAD_DECAY ? head_g : decay[(t * H + h) * d + cc];
       pk[it] = ok ? kv : 0.f;
       pq[it] = ok ? (DELTA ? qv : qv * q_scale) : 0.f;
       pg[it] = ok ? gv : 1.f;
@@ -225,7 +221,7 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
       const bool ok = e < TC * CB && t0 + tok < n && blockIdx.z * CB + c < dv;
       const int64_t t = first + t0 + (ok ? tok : 0);
       const float vv = to_f32(qkv[t * ld + v_col + (int64_t)h * dv + (ok ? blockIdx.z * CB + c : 0)]);
-      pv[it] = ok ? (in_act ? silu_f(vv) : vv) : 0.f;
+      pv[it] = ok ? vv : 0.f;
     }
     if (DELTA && tid < TC) {
       const bool ok = t0 + tid < n;
@@ -340,6 +336,57 @@ __global__ __launch_bounds__(64) void delta_out_kernel(elem_t* __restrict__ y, i
     for (int64_t c = (int64_t)H * dv + threadIdx.x; c < ldy; c += 64) y[(int64_t)t * ldy + c] = from_f32<elem_t>(0.f);
 }
 
+// y[t, :] = o[t, :] / sqrt(mean(o[t, :]^2) + eps) * w * sigmoid(gate[t, :]) (gate_kind 1: * silu) over rows of n entries: one
+// norm for all heads of a read-out.  One workgroup a row; thread t owns the groups of four entries t, t + 256, ... (n in
+// whole groups; a single entry a thread otherwise), sums their squares in that order, a butterfly over the wave follows and
+// the four waves' sums are added in wave order.  The columns of y beyond n are set to zero.
+template <int V>
+__global__ __launch_bounds__(256) void gated_row_norm_kernel(elem_t* __restrict__ y, int64_t ldy, const float* __restrict__ o,
+                                                             const elem_t* __restrict__ gate, int64_t ldg, const void* __restrict__ w, int w_is_f32,
+                                                             int n, float eps, int gate_kind) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const float* row = o + (int64_t)t * n;
+  float part = 0.f;
+  for (int c = threadIdx.x * V; c < n; c += 256 * V) {
+#pragma unroll
+    for (int j = 0; j < V; ++j) part = part + row[c + j] * row[c + j];
+  }
+  part = wave_sum_xor(part);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
+  __syncthreads();
+  const float rr = rsqrtf((((red[0] + red[1]) + red[2]) + red[3]) / (float)n + eps);
+  for (int c = threadIdx.x * V; c < n; c += 256 * V) {
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const float gz = to_f32(gate[(int64_t)t * ldg + c + j]);
+      y[(int64_t)t * ldy + c + j] = from_f32<elem_t>(((row[c + j] * rr) * load_weight(w, w_is_f32, c + j)) * (gate_kind == 0 ? sigmoid_f(gz) : silu_f(gz)));
+    }
+  }
+  for (int64_t c = n + threadIdx.x; c < ldy; c += 256) y[(int64_t)t * ldy + c] = from_f32<elem_t>(0.f);
+}
+
+// x[t, col0 : col0 + n] <- silu(x[t, col0 : col0 + n]) in place, in 32-bit, stored as elements: the activation of a projection
+// whose outputs feed a recurrence.  A thread takes a 16-byte vector where rows and columns are whole vectors (vec).
+__global__ __launch_bounds__(256) void silu_columns_kernel(elem_t* x, int64_t ld, int64_t col0, int n, int T, int vec) {
+  const int per = vec ? n / VK_VEC : n;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)T * per) return;
+  const int64_t t = i / per;
+  const int c = (int)(i - t * per);
+  if (vec) {
+    float v[VK_VEC];
+    elem_t* p = x + t * ld + col0 + (int64_t)c * VK_VEC;
+    load_elems(p, v);
+#pragma unroll
+    for (int j = 0; j < VK_VEC; ++j) v[j] = silu_f(v[j]);
+    store_elems(p, v);
+  } else {
+    elem_t* p = x + t * ld + col0 + c;
+    *p = from_f32<elem_t>(silu_f(to_f32(*p)));
+  }
+}
+
 extern "C" {
 
 // Key channels a lane holds, and lanes that share a value column, for key size d.
@@ -413,12 +460,12 @@ int vk_delta_prep(float* x, int64_t ld, int q_col, int k_col, int T, int G, int 
 // v_col; decay [T, H, d] floats; b: elements, beta's pre-activation of head h at b[t * ldb + h].  state: per slot,
 // the H states at its start, each [dv][d].
 extern "C++" {
-template <bool DELTA, typename IN>
+template <bool DELTA, typename IN, bool HEAD_DECAY = false>
 static int rule_launch(float* out, const IN* qkv, int64_t ld, int q_col, int k_col, int v_col, const float* decay, const elem_t* b, int64_t ldb,
                        float* state, int64_t state_stride, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int G,
-                       int d, int dv, float q_scale, hipStream_t st, const float* head_decay = nullptr, int in_act = 0) {
+                       int d, int dv, float q_scale, hipStream_t st) {
   VK_REQUIRE(S >= 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0, "delta rule: bad sizes H=%d G=%d d=%d dv=%d", H, G, d, dv);
-  VK_REQUIRE((decay != nullptr) != (head_decay != nullptr), "delta rule: decays per token and channel, or one a head");
+  VK_REQUIRE(decay != nullptr, "delta rule: the decays are missing");
   VK_REQUIRE(d <= 1024, "delta rule: key size %d exceeds 1024", d);
   VK_REQUIRE(state_stride >= (int64_t)H * d * dv, "delta rule: the state is too small");
   if (S == 0) return 0;
@@ -427,7 +474,7 @@ static int rule_launch(float* out, const IN* qkv, int64_t ld, int q_col, int k_c
   const dim3 grid(S, H, (dv + cols - 1) / cols);
   VK_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "delta rule: too many heads or columns");
 #define RULE(RR, DD) \
-  delta_rule_kernel<RR, DD, DELTA, IN><<<grid, RULE_THREADS, 0, st>>>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, H, G, d, dv, q_scale, head_decay, in_act)
+  delta_rule_kernel<RR, DD, DELTA, IN, HEAD_DECAY><<<grid, RULE_THREADS, 0, st>>>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, H, G, d, dv, q_scale)
   if (DR == 4) {
     switch (R) {
       case 1: RULE(1, 4); break;
@@ -473,14 +520,34 @@ int vk_gla_rule(float* out, const elem_t* x, int64_t ld, int q_col, int k_col, i
                                     q_scale, st);
 }
 
-// Linear attention with one fixed decay a head: S <- decay[h] S + k v^T, o = S^T q with q = silu(.), k = silu(.), v = silu(.)
-// of the elements at the three columns of x (in_act 1; 0: the elements as they are), q times q_scale.  decay [H] floats.
-int vk_linear_rule(float* out, const elem_t* x, int64_t ld, int q_col, int k_col, int v_col, const float* head_decay, int in_act, float* state,
+// Linear attention with one fixed decay a head: S <- decay[h] S + k v^T, o = S^T (q * q_scale), with q, k (H heads of d) and v
+// (H heads of dv) the elements at the three columns of x.  head_decay [H] floats.
+int vk_linear_rule(float* out, const elem_t* x, int64_t ld, int q_col, int k_col, int v_col, const float* head_decay, float* state,
                    int64_t state_stride, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int d, int dv, float q_scale,
                    hipStream_t st) {
-  VK_REQUIRE(head_decay != nullptr && (in_act == 0 || in_act == 1), "linear attention: the heads' decays are missing");
-  return rule_launch<false, elem_t>(out, x, ld, q_col, k_col, v_col, nullptr, nullptr, 0, state, state_stride, cu_q, positions, slots, S, H, H, d, dv,
-                                    q_scale, st, head_decay, in_act);
+  VK_REQUIRE(head_decay != nullptr, "linear attention: the heads' decays are missing");
+  return rule_launch<false, elem_t, true>(out, x, ld, q_col, k_col, v_col, head_decay, nullptr, 0, state, state_stride, cu_q, positions, slots, S, H, H, d,
+                                          dv, q_scale, st);
+}
+
+// y [T, ldy] elements from o [T, n] floats, gate rows of length ldg and w [n]: gated_row_norm_kernel.
+int vk_gated_row_norm(elem_t* y, int64_t ldy, const float* o, const elem_t* gate, int64_t ldg, const void* w, int w_is_f32, int T, int n, float eps,
+                      int gate_kind, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && n > 0 && ldg >= n && ldy >= n && (gate_kind == 0 || gate_kind == 1), "gated row norm: bad sizes T=%d n=%d", T, n);
+  if (T == 0) return 0;
+  if (n % 4 == 0) gated_row_norm_kernel<4><<<T, 256, 0, st>>>(y, ldy, o, gate, ldg, w, w_is_f32, n, eps, gate_kind);
+  else gated_row_norm_kernel<1><<<T, 256, 0, st>>>(y, ldy, o, gate, ldg, w, w_is_f32, n, eps, gate_kind);
+  return vk_check_launch("gated row norm");
+}
+
+// silu in place on the columns [col0, col0 + n) of x [T, ld].
+int vk_silu_columns(elem_t* x, int64_t ld, int64_t col0, int n, int T, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && n > 0 && col0 >= 0 && ld >= col0 + n, "silu of columns: bad sizes T=%d n=%d", T, n);
+  if (T == 0) return 0;
+  const int vec = n % VK_VEC == 0 && ld % VK_VEC == 0 && col0 % VK_VEC == 0 && (uintptr_t)x % 16 == 0;
+  const int64_t total = (int64_t)T * (vec ? n / VK_VEC : n);
+  silu_columns_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(x, ld, col0, n, T, vec);
+  return vk_check_launch("silu of columns");
 }
 
 int vk_delta_out(elem_t* y, int64_t ldy, const float* o, const elem_t* gate, int64_t ldg, const void* w, int w_is_f32, int T, int H, int dv,

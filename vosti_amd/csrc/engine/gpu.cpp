@@ -149,8 +149,10 @@ struct Kernels::Fn {
   int (*gemm_heads)(P, int64_t, int64_t, CP, int64_t, int64_t, CP, int, int, int, int, hipStream_t);
   int (*latent_post)(CP, int64_t, CP, int64_t, int64_t, int, P, P, P, CP, int, float, CP, int, CP, CP, int, int, int, int, int, int, hipStream_t);
   int (*qkv_post_norm_angles_paired)(CP, int64_t, P, P, P, CP, CP, int, int, float, CP, float, int, int, CP, CP, int, int, int, int, int, hipStream_t);
-  int (*linear_rule)(P, CP, int64_t, int, int, int, CP, int, P, int64_t, CP, CP, CP, int, int, int, int, float, hipStream_t);
+  int (*linear_rule)(P, CP, int64_t, int, int, int, CP, P, int64_t, CP, CP, CP, int, int, int, int, float, hipStream_t);
   int (*side_gate)(P, int64_t, CP, int64_t, CP, int64_t, CP, int, int, int, hipStream_t);
+  int (*gated_row_norm)(P, int64_t, CP, CP, int64_t, CP, int, int, int, float, int, hipStream_t);
+  int (*silu_columns)(P, int64_t, int64_t, int, int, hipStream_t);
 };
 
 static constexpr int KERNEL_ABI = 18;
@@ -195,6 +197,7 @@ Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(na
   VK(cast_from_f32, "vk_cast_from_f32"); VK(moe_route_scored, "vk_moe_route_scored"); VK(moe_glu_weighed, "vk_moe_glu_weighed");
   VK(norm_columns, "vk_norm_columns"); VK(gemm_heads, "vk_gemm_heads"); VK(latent_post, "vk_latent_post");
   VK(qkv_post_norm_angles_paired, "vk_qkv_post_norm_angles_paired"); VK(linear_rule, "vk_linear_rule"); VK(side_gate, "vk_side_gate");
+  VK(gated_row_norm, "vk_gated_row_norm"); VK(silu_columns, "vk_silu_columns");
 #undef VK
   segment_keys_ = fn_->attn_segment_keys();
   item_rows_ = fn_->attn_item_rows();
@@ -1071,7 +1074,7 @@ Tensor Kernels::qkv_post_norm_angles_paired(const Tensor& qkv, int nq, int nkv, 
   return q_out;
 }
 
-Tensor Kernels::linear_rule(const Tensor& x, int64_t q_col, int64_t k_col, int64_t v_col, const Tensor& head_decay, bool silu_inputs, Tensor& state,
+Tensor Kernels::linear_rule(const Tensor& x, int64_t q_col, int64_t k_col, int64_t v_col, const Tensor& head_decay, Tensor& state,
                             const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H, int d, int dv, float q_scale) {
   expect(x, "linear attention input", dtype_);
   expect(state, "state", DType::F32);
@@ -1084,9 +1087,28 @@ Tensor Kernels::linear_rule(const Tensor& x, int64_t q_col, int64_t k_col, int64
   expect(cu_q, "cu_q", DType::I32, {S + 1});
   expect(slots, "state slots", DType::I32, {S});
   Tensor out = empty({T, H, dv}, DType::F32);
-  call(fn_->linear_rule(out.data, x.data, x.dim(1), (int)q_col, (int)k_col, (int)v_col, head_decay.data, silu_inputs ? 1 : 0, state.data, state.dim(1),
+  call(fn_->linear_rule(out.data, x.data, x.dim(1), (int)q_col, (int)k_col, (int)v_col, head_decay.data, state.data, state.dim(1),
                         cu_q.data, positions.data, slots.data, (int)S, H, d, dv, q_scale, stream));
   return out;
+}
+
+Tensor Kernels::gated_row_norm(const Tensor& o, const Tensor& gate, int64_t gate_col, const Tensor& w, float eps, int gate_kind, int64_t width) {
+  expect(o, "read-out", DType::F32);
+  expect(gate, "gate", dtype_);
+  const int64_t T = o.shape.empty() ? 0 : o.dim(0), n = T ? o.numel() / T : 0;
+  if (o.shape.size() < 2 || gate.shape.size() != 2 || gate.dim(0) != T || gate_col < 0 || gate_col + n > gate.dim(1) || width < n || n < 1)
+    throw EngineError("gated row norm: " + o.describe() + " with gate " + gate.describe());
+  const int wf = norm_weight(w, "read-out norm weight", n);
+  Tensor y = empty({T, width});
+  call(fn_->gated_row_norm(y.data, width, o.data, static_cast<const char*>(gate.data) + (size_t)gate_col * dtype_bytes(dtype_), gate.dim(1), w.data, wf,
+                           (int)T, (int)n, eps, gate_kind, stream));
+  return y;
+}
+
+void Kernels::silu_columns(Tensor& x, int64_t first, int64_t count) {
+  expect(x, "rows to activate", dtype_);
+  if (x.shape.size() != 2 || first < 0 || count < 1 || first + count > x.dim(1)) throw EngineError("silu of columns " + std::to_string(first) + ".. of " + x.describe());
+  call(fn_->silu_columns(x.data, x.dim(1), first, (int)count, (int)x.dim(0), stream));
 }
 
 Tensor Kernels::side_gate(const Tensor& gate, const Tensor& table, const Tensor& ids, int64_t first, int64_t n) {

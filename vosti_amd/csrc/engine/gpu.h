@@ -252,9 +252,14 @@ class Kernels {
                                      const Tensor* q_w, const Tensor* k_w, int norm_d, float eps, const Tensor& inv_freq, float mag, bool neighbours,
                                      const Tensor& positions, const Tensor* slots);
   // ---- linear attention with one fixed decay a head (delta.hip)
-  // S <- decay[h] S + k v^T, o = S^T q; silu_inputs: q, k and v pass silu first.  decay [H] floats.  Returns o [T, H, dv] floats.
-  Tensor linear_rule(const Tensor& x, int64_t q_col, int64_t k_col, int64_t v_col, const Tensor& head_decay, bool silu_inputs, Tensor& state,
+  // S <- decay[h] S + k v^T, o = S^T (q * q_scale) from the elements at the three columns of x.  decay [H] floats.  Returns o [T, H, dv] floats.
+  Tensor linear_rule(const Tensor& x, int64_t q_col, int64_t k_col, int64_t v_col, const Tensor& head_decay, Tensor& state,
                      const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H, int d, int dv, float q_scale);
+  // norm(o rows as a whole) * w * act(gate[:, gate_col : gate_col + n]) as elements [T, width] (zero beyond n); o: floats [T, ...] of n
+  // entries a row; gate_kind 0: the logistic function, 1: z * logistic(z).
+  Tensor gated_row_norm(const Tensor& o, const Tensor& gate, int64_t gate_col, const Tensor& w, float eps, int gate_kind, int64_t width);
+  // x[:, first : first + count] <- silu(.) in place.
+  void silu_columns(Tensor& x, int64_t first, int64_t count);
   // ---- a token's slice of a second embedding table, gated (stream.hip)
   // gelu(gate[:, 0:n]) * table[ids, first : first + n] as elements [T, gate.dim(1)], zero beyond n.
   Tensor side_gate(const Tensor& gate, const Tensor& table, const Tensor& ids, int64_t first, int64_t n);

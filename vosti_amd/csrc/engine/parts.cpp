@@ -1449,8 +1449,9 @@ class LatentAttention : public Mixer {
 //   y = norm(the heads' o side by side) (one root mean square over all of them, a weight of that width) * sigmoid(W_g h);
 //   out = W_o y.
 // A request's state slot holds the heads' S in 32-bit, zero at the request's start.  The four input projections are one
-// launch; the recurrence is the delta rule's walk without its correction term, with the decays of the heads (numbers
-// decay.0, decay.1, ...) in place of decays per token and channel; the read-out's norm and gate are one launch.
+// launch, silu on its q, k and v columns a second; the recurrence is the delta rule's walk without its correction term, with
+// the decays of the heads (numbers decay.0, decay.1, ...) in place of decays per token and channel; the read-out's norm and
+// gate are one launch, a workgroup a row.
 class FixedDecayAttention : public Mixer {
  public:
   FixedDecayAttention(const PartSpec& s, Kernels& k)
@@ -1487,11 +1488,11 @@ class FixedDecayAttention : public Mixer {
   Tensor forward(const Tensor& x, StepContext& ctx, CacheEntry& cache) override {
     if (cache.kind != CacheNeed::State) throw EngineError("linear attention was handed a cache entry without state");
     Kernels& k = kernels;
-    const Tensor proj = k.gemm(x, w_in_);
-    const Tensor o = k.linear_rule(proj, 0, qk_, 2 * qk_, decay_, true, cache.state, ctx.cu_q, ctx.positions, ctx.state_slots, H_, d_, dv_, 1.f);
-    // One norm over all heads: the read-out as one head of H * dv entries.
-    const Tensor all = o.view({o.dim(0), 1, (int64_t)H_ * dv_});
-    return k.gemm(k.gated_head_norm(all, proj, 2 * qk_ + v_, out_norm_, 1, H_ * dv_, eps_, 0, v_), w_o_);
+    Tensor proj = k.gemm(x, w_in_);
+    // q, k and v pass silu once, in place (the recurrence's workgroups would each do it again for the columns they share).
+    k.silu_columns(proj, 0, 2 * qk_ + v_);
+    const Tensor o = k.linear_rule(proj, 0, qk_, 2 * qk_, decay_, cache.state, ctx.cu_q, ctx.positions, ctx.state_slots, H_, d_, dv_, 1.f);
+    return k.gemm(k.gated_row_norm(o, proj, 2 * qk_ + v_, out_norm_, eps_, 0, v_), w_o_);
   }
 
  private:

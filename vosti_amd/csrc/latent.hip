@@ -13,25 +13,30 @@
 #include "mma.h"
 #include "vec.h"
 
-// One wave a row: y[t, 0:n] = norm(x[t, col : col + n]) * w, y[t, n:ldy] = 0.  The sum of squares runs over a lane's
-// elements l, l + 64, ... in order and then as a butterfly.
+// One workgroup a row: y[t, 0:n] = norm(x[t, col : col + n]) * w, y[t, n:ldy] = 0.  The sum of squares runs over a thread's
+// elements t, t + 256, ... in order, then as a butterfly over a wave, and the four waves' sums are added in wave order: the
+// order depends on n alone.
 __global__ __launch_bounds__(256) void norm_columns_kernel(elem_t* __restrict__ y, int64_t ldy, const elem_t* __restrict__ x, int64_t ldx, int col,
-                                                           int n, const void* __restrict__ w, int w_is_f32, float eps, int T) {
-  const int lane = threadIdx.x & 63, t = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (t >= T) return;
+                                                           int n, const void* __restrict__ w, int w_is_f32, float eps) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
   const elem_t* row = x + (int64_t)t * ldx + col;
   float part = 0.f;
-  for (int c = lane; c < n; c += 64) {
+  for (int c = threadIdx.x; c < n; c += 256) {
     const float v = to_f32(row[c]);
     part = part + v * v;
   }
-  const float rr = rsqrtf(wave_sum_xor(part) / (float)n + eps);
-  for (int c = lane; c < ldy; c += 64)
+  part = wave_sum_xor(part);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
+  __syncthreads();
+  const float rr = rsqrtf((((red[0] + red[1]) + red[2]) + red[3]) / (float)n + eps);
+  for (int c = threadIdx.x; c < ldy; c += 256)
     y[(int64_t)t * ldy + c] = from_f32<elem_t>(c < n ? (to_f32(row[c]) * rr) * load_weight(w, w_is_f32, c) : 0.f);
 }
 
 // out[t, h * os + f] = sum over k < K of w[h][f][k] * x[t, h * xs + k] for f < N: a product a head, its weights [H, N, K].
-// A workgroup of four waves takes 16 rows, one head and 64 output features (16 a wave).  The sums have the order of this
+// A wave takes 16 rows and 64 output features of one head (four accumulators that share the rows' fragments); a workgroup's
+// four waves take four such row tiles side by side, so that they read the same weights.  The sums have the order of this
 // library's other products: the reduction axis in chunks of 512 elements, a chunk's products added from zero over ascending
 // slabs of 64 bytes with the weights as first operand, the chunk sums added to a zero total in chunk order.
 #define HEADS_KC 512
@@ -39,29 +44,49 @@ __global__ __launch_bounds__(256) void gemm_heads_kernel(elem_t* __restrict__ ou
                                                          int64_t xs, const elem_t* __restrict__ w, int T, int N, int K) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kq = lane >> 4;
-  const int f0 = blockIdx.x * 64 + wave * 16, t0 = blockIdx.y * 16, h = blockIdx.z;
-  if (f0 >= N) return;
-  const bool w_ok = f0 + r16 < N, x_ok = t0 + r16 < T;
-  const elem_t* wr = w + ((int64_t)h * N + (w_ok ? f0 + r16 : 0)) * K + kq * VK_VEC;
+  const int f0 = blockIdx.x * 64, t0 = (blockIdx.y * 4 + wave) * 16, h = blockIdx.z;
+  if (t0 >= T) return;
+  const bool x_ok = t0 + r16 < T;
   const elem_t* xr = x + (int64_t)(x_ok ? t0 + r16 : 0) * ldx + (int64_t)h * xs + kq * VK_VEC;
-  f32x4 total = {0.f, 0.f, 0.f, 0.f};
+  const elem_t* wr[4];
+  bool w_ok[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    w_ok[j] = f0 + 16 * j + r16 < N;
+    wr[j] = w + ((int64_t)h * N + (w_ok[j] ? f0 + 16 * j + r16 : 0)) * K + kq * VK_VEC;
+  }
+  f32x4 total[4], acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) total[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int c0 = 0; c0 < K; c0 += HEADS_KC) {
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int end = min(K, c0 + HEADS_KC);
-#pragma unroll 4
+#pragma unroll 2
     for (int k = c0; k < end; k += VK_SLAB) {
       const bool k_ok = k + kq * VK_VEC < K;
-      acc = mma_slab(load_frag(wr + k, w_ok && k_ok), load_frag(xr + k, x_ok && k_ok), acc);
+      const frag_t fx = load_frag(xr + k, x_ok && k_ok);
+      frag_t fw[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) fw[j] = load_frag(wr[j] + k, w_ok[j] && k_ok);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = mma_slab(fw[j], fx, acc[j]);
     }
-    total.x = total.x + acc.x; total.y = total.y + acc.y; total.z = total.z + acc.z; total.w = total.w + acc.w;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      total[j].x = total[j].x + acc[j].x; total[j].y = total[j].y + acc[j].y; total[j].z = total[j].z + acc[j].z; total[j].w = total[j].w + acc[j].w;
+    }
   }
-  // Lane l holds features f0 + 4 * (l / 16) + i of row l % 16.
+  // Lane l holds features f0 + 16 j + 4 * (l / 16) + i of row l % 16.
   if (!x_ok) return;
   elem_t* o = out + (int64_t)(t0 + r16) * ldo + (int64_t)h * os;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int f = f0 + kq * 4 + i;
-    if (f < N) o[f] = from_f32<elem_t>(total[i]);
+  for (int j = 0; j < 4; ++j) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int f = f0 + 16 * j + kq * 4 + i;
+      if (f < N) o[f] = from_f32<elem_t>(total[j][i]);
+    }
   }
 }
 
@@ -141,7 +166,7 @@ int vk_norm_columns(elem_t* y, int64_t ldy, const elem_t* x, int64_t ldx, int co
                     hipStream_t st) {
   VK_REQUIRE(T >= 0 && n > 0 && col >= 0 && ldx >= (int64_t)col + n && ldy >= n, "norm of columns: bad sizes T=%d n=%d col=%d", T, n, col);
   if (T == 0) return 0;
-  norm_columns_kernel<<<(T + 3) / 4, 256, 0, st>>>(y, ldy, x, ldx, col, n, w, w_is_f32, eps, T);
+  norm_columns_kernel<<<T, 256, 0, st>>>(y, ldy, x, ldx, col, n, w, w_is_f32, eps);
   return vk_check_launch("norm of columns");
 }
 
@@ -153,9 +178,9 @@ int vk_gemm_heads(elem_t* out, int64_t ldo, int64_t os, const elem_t* x, int64_t
              "product a head: bad sizes H=%d N=%d K=%d (K and the input's strides in whole 16-byte vectors)", H, N, K);
   VK_REQUIRE(ldx >= (int64_t)(H - 1) * xs + K && ldo >= (int64_t)(H - 1) * os + N && os >= 0 && xs >= 0, "product a head: the rows do not hold the heads");
   VK_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "product a head: operands must be 16-byte aligned");
-  VK_REQUIRE(H <= 65535 && (T + 15) / 16 <= 65535, "product a head: too many heads or rows for one launch");
+  VK_REQUIRE(H <= 65535 && (T + 63) / 64 <= 65535, "product a head: too many heads or rows for one launch");
   if (T == 0) return 0;
-  gemm_heads_kernel<<<dim3((N + 63) / 64, (T + 15) / 16, H), 256, 0, st>>>(out, ldo, os, x, ldx, xs, w, T, N, K);
+  gemm_heads_kernel<<<dim3((N + 63) / 64, (T + 63) / 64, H), 256, 0, st>>>(out, ldo, os, x, ldx, xs, w, T, N, K);
   return vk_check_launch("product a head");
 }
 
