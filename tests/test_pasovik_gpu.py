@@ -400,6 +400,22 @@ def test_greedy_generation_through_the_scheduler(models, graphs):
         assert list(got) == plain.generate_greedy(cfg, w, prompt, 12)
 
 
+def test_the_command_line_generates_the_plain_tokens(models):
+    """The engine's program, started as a user starts it with --family pasovik: greedy tokens of the plain implementation."""
+    import json
+    import subprocess
+    from vosti_amd.kernels import build
+    folder, cfg, w = models["MIXED"]
+    program = str(build.ensure("engine", verbose=False))
+    lib = build.ensure("f32", verbose=False)
+    prompt = tokens_for(cfg, 21, 70)
+    r = subprocess.run([program, "--family", "pasovik", "--dtype", "float32", "--lib-dir", str(lib.parent), "--model-path", str(folder),
+                        "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "8", "--page-size", "16"], capture_output=True, text=True, timeout=110, env={})
+    assert r.returncode == 0, r.stderr[-2000:]
+    out = json.loads([l for l in r.stdout.splitlines() if l.startswith("MODEL_OUTPUT_TOKEN_IDS=")][0].split("=", 1)[1])
+    assert out == plain.generate_greedy(cfg, w, prompt, 8)
+
+
 # --------------------------------------------------------------------------------------------- the replay program
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_the_replay_program_with_four_slots_and_a_pool_for_the_live_requests(models, tmp_path, dtype):
