@@ -147,17 +147,30 @@ def test_a_weight_scales_what_an_expert_reads(tmp_path):
 
 
 def test_the_residual_stream_is_32_bit(tmp_path):
-    """Many layers with small updates on a large embedding: a stream rounded to 16 bits between layers would lose them."""
-    cfg = config([layer("lightning", SMALL_MIXER, None) for _ in range(12)], width=32, vocab=40)
+    """Sixteen layers with the same weights add the same small update sixteen times to a large embedding; each update is below
+    half a step of a 16-bit stream of that size, so a stream that is rounded to 16 bits between sublayers loses them all.
+    The plain implementation with such a stream is checked to be far off first; the engine must be near the true one."""
+    cfg = config([layer("lightning", SMALL_MIXER, None) for _ in range(16)], width=32, vocab=40)
     w = random_weights(cfg, 5)
-    for n in w:
-        if n.endswith("norm1"):
-            w[n] = torch.full_like(w[n], 0.05)
-    w["embed"] = (w["embed"].float() * 40.0).to(torch.bfloat16)
-    folder = write_model(tmp_path / "deep", cfg, w)
+    for n in list(w):
+        if n.startswith("l0."):
+            for i in range(1, 16):
+                w[f"l{i}." + n[3:]] = w[n].clone()
+    for i in range(16):
+        w[f"l{i}.norm1"] = torch.full_like(w[f"l{i}.norm1"], 0.1)
+    w["embed"] = (torch.sign(w["embed"].float()) * (32.0 + 16.0 * torch.rand(w["embed"].shape, generator=torch.Generator().manual_seed(1)))).to(torch.bfloat16)
     tokens = tokens_for(cfg, 20, 2)
+    want = plain_logits(cfg, w, tokens)
+    # The plain layers once more with a stream that is rounded to bfloat16 after every add.
+    x = w["embed"].double()[torch.tensor(tokens)]
+    for i in range(16):
+        y, _ = plain.lightning(cfg["layers"][i]["mixer"], w, f"l{i}.mix.", x, cfg["norm"]["eps"])
+        x = (x + plain.norm(y, w[f"l{i}.norm1"], cfg["norm"]["eps"])).to(torch.bfloat16).double()
+    lossy = (plain.norm(x, w["final.norm"], cfg["norm"]["eps"]) @ w["head"].double().T).numpy()
+    assert deviation(lossy, want) > 2.5e-2
+    folder = write_model(tmp_path / "deep", cfg, w)
     got = run_cut(engine(folder, "bfloat16"), 0, tokens, [20])
-    assert deviation(got, plain_logits(cfg, w, tokens)) < 1.5e-2
+    assert deviation(got, want) < 1.0e-2
 
 
 # ----------------------------------------------------------------------------- cuttings, batches, pages and slots
