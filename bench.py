@@ -591,8 +591,8 @@ def pasovik_config(width, heads, kv_heads, ff, layers, vocab):
             out.append({"type": "lightning", "mixer": {"dim": 128, "vdim": 128, "heads": heads, "decay": decay}, "mlp": dense})
         elif kind == 1:
             out.append({"type": "attention", "mlp": experts,
-                        "mixer": {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": kv_heads, "scale": 128 ** -0.5, "softcap": 20.0,
-                                  "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0}}}})
+                        "mixer": {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": kv_heads, "scale": 128 ** -0.5, "softcap": 30.0,
+                                  "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0}}}})
         else:
             out.append({"type": "latent_attention", "mixer": latent(i - 1 if kind == 3 else None), "mlp": dense if kind == 2 else experts})
     return {"architecture": "Pasovik", "layers": out, "norm": {"eps": 1e-5}, "token_side": {"dim": 256}, "vocab": vocab, "width": width}

@@ -71,9 +71,9 @@ MIXED = config([
     layer("latent_attention", latent(1, 24, 16, 24, kv_rank=48, q_rank=8, factor=8.0, kv_from=6), moe(5, 2, 24, limit=1.0)),
 ], width=64, vocab=97, side=5)
 # The head size of the kernels' widest tiles, a cache row of a latent as wide, and a state as wide as a wave; no side input.
-WIDE = config([layer("attention", attention(4, 2, 128, 128, rot_dims=32, base=250000.0, softcap=30.0), moe(12, 5, 64, limit=1.25)),
+WIDE = config([layer("attention", attention(4, 2, 128, 128, rot_dims=32, base=400000.0, softcap=30.0), moe(12, 5, 64, limit=1.25)),
                layer("lightning", lightning(2, 64, 64, [0.9, 0.99]), dense(120)),
-               layer("latent_attention", latent(4, 32, 16, 32, kv_rank=112, q_rank=48, base=250000.0), dense(64))], width=96, vocab=130)
+               layer("latent_attention", latent(4, 32, 16, 32, kv_rank=112, q_rank=48, base=400000.0), dense(64))], width=96, vocab=130)
 CONFIGS = {"MIXED": MIXED, "WIDE": WIDE}
 
 

@@ -107,7 +107,7 @@ def test_tensor_names_are_the_files(tmp_path):
 
 def test_the_rotation_frequencies_are_the_plain_ones():
     from vosti_amd.cache.host import rotary_linear_frequencies
-    for base, dims, factor in ((10000.0, 8, None), (250000.0, 48, 4.0), (77.0, 2, 2.5)):
+    for base, dims, factor in ((10000.0, 8, None), (400000.0, 40, 3.0), (77.0, 2, 2.5)):
         rot = {"base": base, "dims": dims}
         if factor:
             rot["scaling"] = {"factor": factor}
