@@ -80,7 +80,9 @@ ALONE = {
     "attention_wide_values": config([layer("attention", attention(2, 2, 8, 48, rot_dims=4), None)], width=32, vocab=50),
     "attention_keys_wider_than_values": config([layer("attention", attention(3, 3, 40, 24, rot_dims=20, softcap=50.0), None)], width=32, vocab=50),
     "attention_one_head_one_pair": config([layer("attention", attention(1, 1, 16, 16, rot_dims=2, scale=1.0), None)], width=32, vocab=50),
+    "attention_many_heads_on_one_key_head": config([layer("attention", attention(24, 1, 16, 16, rot_dims=8), None)], width=32, vocab=50),
     "latent": config([layer("latent_attention", latent(3, 16, 8, 16, kv_rank=24, q_rank=16), None)], width=32, vocab=50),
+    "latent_twenty_heads": config([layer("latent_attention", latent(20, 8, 4, 8, kv_rank=16, q_rank=16), None)], width=32, vocab=50),
     "latent_odd_sizes": config([layer("latent_attention", latent(5, 10, 6, 12, kv_rank=13, q_rank=11, base=300.0, factor=2.5), None)], width=32, vocab=50),
     "latent_one_head_wide": config([layer("latent_attention", latent(1, 64, 32, 80, kv_rank=96, q_rank=40), None)], width=32, vocab=50),
     "latent_values_wider_than_the_latent": config([layer("latent_attention", latent(2, 8, 2, 40, kv_rank=8, q_rank=8), None)], width=32, vocab=50),
